@@ -1,0 +1,134 @@
+/*
+ * lutgemm_gfx950.h -- C ABI of the MI355X (gfx950) LUT-GEMM engine for
+ * binary-coding-quantised (BCQ) linear layers.
+ *
+ * This is the boundary a host binding sits on: plain pointers and sizes, no
+ * torch types.  All pointers are DEVICE pointers on the current HIP device;
+ * `stream` is a hipStream_t passed as void* (NULL = the null stream).  Every
+ * call is asynchronous with respect to the host and returns 0 on success or a
+ * negative LUTGEMM_E* code; nothing throws and nothing is printed.
+ *
+ * Shared operand conventions (paths are relative to the ShiftAddLLM
+ * reference checkout):
+ *   N = out features ("mSize"), K = in features ("kSize"), nb = bit planes.
+ *   bW    : uint32 [K/32][nb][N]; bit t of bW[w][b][n] set <=> sign
+ *           B[n][32w+t][b] = +1; byte j of the word indexes the 256-entry
+ *           table of inputs 32w+8j .. 32w+8j+7
+ *           (lut_gemm/mv_fp16_bias.hpp:19-26,52,86-90; lut_gemm/quant.py:25).
+ *   x     : fp16 [M][K] row-major (row m at x + m*K).
+ *   out   : fp16 [M][N] row-major.  The engine ACCUMULATES: out += W_q x,
+ *           the caller pre-fills out with the bias or zeros
+ *           (mv_fp16_bias.hpp:101,216,324,491,577; lut_gemm/quant.py:46).
+ *           Unlike the reference's fp16 atomics the sum is formed in fp32 and
+ *           rounded to fp16 once, and it is deterministic.
+ * Shape rules enforced here (the reference checks nothing and reads or writes
+ * out of bounds instead): K % 32 == 0, N % 4 == 0, 1 <= nb <= 4, M >= 1,
+ * 16-byte aligned bW, 8-byte aligned row-wise alpha.
+ */
+#ifndef LUTGEMM_GFX950_H
+#define LUTGEMM_GFX950_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define LUTGEMM_OK 0
+#define LUTGEMM_EINVAL (-1)   /* bad shape / size / null pointer            */
+#define LUTGEMM_EALIGN (-2)   /* pointer not aligned as required            */
+#define LUTGEMM_EUNSUP (-3)   /* legal in the reference API, not built here */
+#define LUTGEMM_EHIP (-4)     /* a HIP runtime call failed                  */
+#define LUTGEMM_ENOMEM (-5)   /* workspace allocation failed                */
+
+/* Human-readable text for a return code (static storage). */
+const char *lutgemm_strerror(int code);
+
+/* HIP error of the last LUTGEMM_EHIP on this thread (hipError_t as int). */
+int lutgemm_last_hip_error(void);
+
+/*
+ * Row-wise alpha, groups along K.
+ * Replaces lutgemm_compute_shift_scale -> nqmv_bias_shift_mulq ->
+ * _nqmv_bias_shift_mulq<32>  (lut_gemm/lutgemm_cuda.cpp:43-52;
+ * lutgemm_cuda_kernel.cu:268-285; mv_fp16_bias.hpp:498-579,766-774).
+ *   alpha : fp16 [num_groups][nb][N], group g covers inputs
+ *           g*(K/num_groups) .. ; K/num_groups must be a multiple of 32.
+ *   out[m][n] += sum_g sum_b alpha[g][b][n] * sum_{k in g} B[n][k][b] x[m][k]
+ * The reference entry point is batch-1; M > 1 rows are a superset.
+ */
+int lutgemm_gemv_rowwise_f16(const uint32_t *bW, const void *alpha_f16, const void *x_f16,
+                             void *out_f16, int N, int K, int nb, int num_groups, int M,
+                             void *stream);
+
+/*
+ * Uniform-quantisation mode of the original LUT-GEMM.
+ * Replaces lutgemm_compute -> nqmv_bias -> _nqmv_bias<32>
+ * (lutgemm_cuda.cpp:88-98; lutgemm_cuda_kernel.cu:287-315;
+ *  mv_fp16_bias.hpp:8-103,726-734).
+ *   alpha, q_bias : fp16 [num_groups][N]
+ *   out[m][n] += sum_g ( q_bias[g][n] * sum_{k in g} x[m][k]
+ *                + sum_b alpha[g][n] / 2^(b+1) * sum_{k in g} B[n][k][b] x[m][k] )
+ */
+int lutgemm_gemv_uniform_f16(const uint32_t *bW, const void *alpha_f16, const void *qbias_f16,
+                             const void *x_f16, void *out_f16, int N, int K, int nb,
+                             int num_groups, int M, void *stream);
+
+/*
+ * Block alpha (ShiftAddLLM "Lat."): one alpha per 8-input chunk, bit plane and
+ * row group.  R = num_groups row groups of N/R consecutive outputs.
+ *   out[m][n] += sum_c sum_b A(c, b, n / (N/R)) * LUT_c[byte(c,b,n)]
+ * (N/R) % 4 == 0 is required.
+ *
+ * _f16      : A = alpha fp16 [K/8][nb][R].  Replaces lutgemm_compute_block ->
+ *             _nqmv_bias_block<32> (lutgemm_cuda.cpp:54-63;
+ *             lutgemm_cuda_kernel.cu:318-346; mv_fp16_bias.hpp:105-220,736-744).
+ * _shift_u16: alpha uint16 [K/8][nb][R] of three 3-bit shift fields,
+ *             A = 2^(u&7) + 2^((u>>3)&7) + 2^((u>>6)&7).  Replaces
+ *             lutgemm_compute_block_shift -> _nqmv_bias_block_shift<32>
+ *             (lutgemm_cuda.cpp:65-74; lutgemm_cuda_kernel.cu:349-377;
+ *             mv_fp16_bias.hpp:223-328,746-754).
+ * _apot_i8  : alpha int8 [K/8][nb][R][3] signed exponents,
+ *             A = 2^s0 + 2^s1 + 2^s2, a term with s = -128 is absent.
+ *             Replaces lutgemm_compute_block_shiftInt8 ->
+ *             _nqmv_bias_block_shiftInt8<32> (lutgemm_cuda.cpp:76-85;
+ *             lutgemm_cuda_kernel.cu:380-408; mv_fp16_bias.hpp:335-340,
+ *             342-495,756-764) -- the call LutLinear.forward makes
+ *             (lut_gemm/quant.py:50-51).
+ * num_apot must be 3: the reference ignores the argument and hard-codes three
+ * terms (mv_fp16_bias.hpp:294,473-482).
+ */
+int lutgemm_gemv_block_f16(const uint32_t *bW, const void *alpha_f16, const void *x_f16,
+                           void *out_f16, int N, int K, int nb, int num_groups, int M,
+                           void *stream);
+int lutgemm_gemv_block_shift_u16(const uint32_t *bW, const uint16_t *alpha_u16, const void *x_f16,
+                                 void *out_f16, int N, int K, int nb, int num_groups,
+                                 int num_apot, int M, void *stream);
+int lutgemm_gemv_block_apot_i8(const uint32_t *bW, const int8_t *alpha_i8, const void *x_f16,
+                               void *out_f16, int N, int K, int nb, int num_groups, int num_apot,
+                               int M, void *stream);
+
+/*
+ * Algorithmic HBM bytes of one call (signs + alphas + x + out read + out
+ * write), the figure throughput is quoted against.  alpha_bytes_per_entry is
+ * 2 (fp16, uint16) or 3 (int8 x 3); alpha_entries is the alpha element count.
+ */
+size_t lutgemm_algorithmic_bytes(int N, int K, int nb, int M, size_t alpha_entries,
+                                 int alpha_bytes_per_entry);
+
+/*
+ * Measurement helper: a plain device-to-device copy of `bytes` (multiple of
+ * 16) done by a kernel of this library, used to calibrate profiler byte
+ * counters against a known traffic.  No counterpart in the reference.
+ */
+int lutgemm_copy_bytes(void *dst, const void *src, size_t bytes, void *stream);
+
+/* Release the per-stream workspaces this library allocated on the current
+ * device (optional; they otherwise live until the process ends). */
+int lutgemm_release_workspaces(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* LUTGEMM_GFX950_H */

@@ -1,0 +1,90 @@
+"""In-tree build of the two native pieces (no JIT cache, no install step).
+
+  liblutgemm_gfx950.so          hipcc --offload-arch=gfx950, kernels + C ABI
+  lutgemm.cpython-*.so          g++, the `lutgemm` Python module (torch shim),
+                                linked against the library above via $ORIGIN
+
+Run `python -m shiftaddllm_amd.build` (add --force to rebuild everything).
+hipcc cross-compiles for gfx950 without a GPU present.
+"""
+from __future__ import annotations
+
+import os
+import subprocess
+import sys
+import sysconfig
+
+PKG_DIR = os.path.dirname(os.path.abspath(__file__))
+REPO_DIR = os.path.dirname(PKG_DIR)
+CSRC = os.path.join(PKG_DIR, "csrc")
+INCLUDE = os.path.join(REPO_DIR, "include")
+ROCM = os.environ.get("ROCM_PATH", "/opt/rocm")
+
+KERNEL_LIB = os.path.join(PKG_DIR, "liblutgemm_gfx950.so")
+EXT_SUFFIX = sysconfig.get_config_var("EXT_SUFFIX") or ".so"
+TORCH_EXT = os.path.join(PKG_DIR, "lutgemm" + EXT_SUFFIX)
+
+# -packed-fp32-ops is switched off for all device code: hipcc would otherwise
+# form v_pk_*_f32 from ordinary float arithmetic.
+HIPCC_FLAGS = [
+    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wno-unused-command-line-argument",
+]
+
+
+def _newer(target: str, *sources: str) -> bool:
+    if not os.path.exists(target):
+        return False
+    t = os.path.getmtime(target)
+    return all(os.path.getmtime(s) <= t for s in sources)
+
+
+def _run(cmd):
+    print("+", " ".join(cmd), flush=True)
+    subprocess.check_call(cmd)
+
+
+def build_kernel_library(force: bool = False) -> str:
+    src = os.path.join(CSRC, "lutgemm_kernels.hip")
+    hdr = os.path.join(INCLUDE, "lutgemm_gfx950.h")
+    if not force and _newer(KERNEL_LIB, src, hdr):
+        return KERNEL_LIB
+    hipcc = os.path.join(ROCM, "bin", "hipcc")
+    _run([hipcc, *HIPCC_FLAGS, "-I", INCLUDE, "-o", KERNEL_LIB, src])
+    return KERNEL_LIB
+
+
+def build_torch_extension(force: bool = False) -> str:
+    src = os.path.join(CSRC, "lutgemm_torch.cpp")
+    hdr = os.path.join(INCLUDE, "lutgemm_gfx950.h")
+    if not force and _newer(TORCH_EXT, src, hdr, KERNEL_LIB):
+        return TORCH_EXT
+    import torch
+    from torch.utils import cpp_extension
+
+    torch_lib = os.path.join(os.path.dirname(torch.__file__), "lib")
+    inc = []
+    for d in cpp_extension.include_paths():
+        inc += ["-isystem", d]
+    inc += ["-isystem", os.path.join(ROCM, "include"), "-isystem", sysconfig.get_paths()["include"]]
+    abi = int(torch.compiled_with_cxx11_abi())
+    cmd = [
+        os.environ.get("CXX", "g++"), "-O2", "-std=c++17", "-fPIC", "-shared",
+        "-DTORCH_EXTENSION_NAME=lutgemm", "-DTORCH_API_INCLUDE_EXTENSION_H",
+        "-DUSE_ROCM=1", "-D__HIP_PLATFORM_AMD__=1", f"-D_GLIBCXX_USE_CXX11_ABI={abi}",
+        "-I", INCLUDE, *inc, src, "-o", TORCH_EXT,
+        "-L", PKG_DIR, "-llutgemm_gfx950",
+        "-L", torch_lib, "-lc10", "-lc10_hip", "-ltorch_cpu", "-ltorch_hip", "-ltorch", "-ltorch_python",
+        "-Wl,-rpath,$ORIGIN", "-Wl,--no-as-needed",
+    ]
+    _run(cmd)
+    return TORCH_EXT
+
+
+def build_all(force: bool = False):
+    return build_kernel_library(force), build_torch_extension(force)
+
+
+if __name__ == "__main__":
+    build_all(force="--force" in sys.argv)

@@ -1,0 +1,97 @@
+"""Loader for the compiled pieces.  Fails loudly: no fallback path exists.
+
+`lutgemm`  -- the CPython module with the reference's call signatures
+              (lut_gemm/lutgemm_cuda.cpp:225-230 in the ShiftAddLLM checkout).
+`cabi()`   -- ctypes handle on liblutgemm_gfx950.so with argtypes set from
+              include/lutgemm_gfx950.h, for callers that bind the C ABI directly.
+"""
+from __future__ import annotations
+
+import ctypes
+import importlib.util
+import os
+import sys
+import sysconfig
+
+_PKG_DIR = os.path.dirname(os.path.abspath(__file__))
+KERNEL_LIB = os.path.join(_PKG_DIR, "liblutgemm_gfx950.so")
+TORCH_EXT = os.path.join(_PKG_DIR, "lutgemm" + (sysconfig.get_config_var("EXT_SUFFIX") or ".so"))
+
+C_ABI_SYMBOLS = (
+    "lutgemm_strerror",
+    "lutgemm_last_hip_error",
+    "lutgemm_gemv_rowwise_f16",
+    "lutgemm_gemv_uniform_f16",
+    "lutgemm_gemv_block_f16",
+    "lutgemm_gemv_block_shift_u16",
+    "lutgemm_gemv_block_apot_i8",
+    "lutgemm_algorithmic_bytes",
+    "lutgemm_copy_bytes",
+    "lutgemm_release_workspaces",
+)
+
+
+class NativeLibraryMissing(ImportError):
+    pass
+
+
+def _missing(path: str) -> NativeLibraryMissing:
+    return NativeLibraryMissing(
+        f"{path} has not been built. Run `python -m shiftaddllm_amd.build` "
+        "(hipcc --offload-arch=gfx950). There is no fallback compute path.")
+
+
+def _load_extension():
+    if not os.path.exists(KERNEL_LIB):
+        raise _missing(KERNEL_LIB)
+    if not os.path.exists(TORCH_EXT):
+        raise _missing(TORCH_EXT)
+    import torch  # noqa: F401  (its HIP runtime must be the one already loaded)
+    spec = importlib.util.spec_from_file_location("lutgemm", TORCH_EXT)
+    module = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(module)
+    # `import lutgemm` elsewhere in the process (the reference's quant.py does
+    # exactly that) now resolves to this module.
+    sys.modules.setdefault("lutgemm", module)
+    return module
+
+
+_cabi = None
+
+
+def cabi() -> ctypes.CDLL:
+    global _cabi
+    if _cabi is None:
+        if not os.path.exists(KERNEL_LIB):
+            raise _missing(KERNEL_LIB)
+        import torch  # noqa: F401
+        lib = ctypes.CDLL(KERNEL_LIB)
+        vp, ci, sz = ctypes.c_void_p, ctypes.c_int, ctypes.c_size_t
+        lib.lutgemm_strerror.argtypes = [ci]
+        lib.lutgemm_strerror.restype = ctypes.c_char_p
+        lib.lutgemm_last_hip_error.argtypes = []
+        lib.lutgemm_last_hip_error.restype = ci
+        lib.lutgemm_gemv_rowwise_f16.argtypes = [vp, vp, vp, vp, ci, ci, ci, ci, ci, vp]
+        lib.lutgemm_gemv_uniform_f16.argtypes = [vp, vp, vp, vp, vp, ci, ci, ci, ci, ci, vp]
+        lib.lutgemm_gemv_block_f16.argtypes = [vp, vp, vp, vp, ci, ci, ci, ci, ci, vp]
+        lib.lutgemm_gemv_block_shift_u16.argtypes = [vp, vp, vp, vp, ci, ci, ci, ci, ci, ci, vp]
+        lib.lutgemm_gemv_block_apot_i8.argtypes = [vp, vp, vp, vp, ci, ci, ci, ci, ci, ci, vp]
+        for name in ("lutgemm_gemv_rowwise_f16", "lutgemm_gemv_uniform_f16", "lutgemm_gemv_block_f16",
+                     "lutgemm_gemv_block_shift_u16", "lutgemm_gemv_block_apot_i8"):
+            getattr(lib, name).restype = ci
+        lib.lutgemm_algorithmic_bytes.argtypes = [ci, ci, ci, ci, sz, ci]
+        lib.lutgemm_algorithmic_bytes.restype = sz
+        lib.lutgemm_copy_bytes.argtypes = [vp, vp, sz, vp]
+        lib.lutgemm_copy_bytes.restype = ci
+        lib.lutgemm_release_workspaces.argtypes = []
+        lib.lutgemm_release_workspaces.restype = ci
+        _cabi = lib
+    return _cabi
+
+
+def __getattr__(name):
+    if name == "lutgemm":
+        module = _load_extension()
+        globals()["lutgemm"] = module
+        return module
+    raise AttributeError(name)

@@ -1,0 +1,297 @@
+"""Parity of the HIP kernels with the CPU oracle, on the GPU, through the C ABI.
+
+Bars: packed words and table indices are bit-exact by construction of the
+operands (checked on the CPU side); outputs are fp16 and must satisfy
+rel-L2 <= 2e-3 and max|dy| <= 1e-2 * max|y_ref| against the oracle.  The
+kernels accumulate in fp32 and round once, so the tests also hold them to a
+ten times tighter bound.
+"""
+import ctypes
+
+import numpy as np
+import pytest
+import torch
+
+import oracle as orc
+from shiftaddllm_amd import native, workload
+
+pytestmark = pytest.mark.gpu
+
+REL_L2_BAR = 2e-3          # relative L2 error bound on the fp16 output
+MAX_ABS_BAR = 1e-2         # max |dy| / max |y_ref|
+TIGHT = 0.1                # our own margin inside those bars
+
+
+def _stream():
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _ptr(t):
+    return ctypes.c_void_p(t.data_ptr())
+
+
+def _check(rc):
+    assert rc == 0, native.cabi().lutgemm_strerror(rc).decode()
+
+
+def _assert_close(y_gpu, y_ref, what=""):
+    rel, mad = orc.error_metrics(y_gpu.float().cpu().numpy(), np.asarray(y_ref, dtype=np.float32))
+    assert rel <= REL_L2_BAR * TIGHT and mad <= MAX_ABS_BAR * TIGHT, (what, rel, mad)
+    return rel, mad
+
+
+def run_rowwise(dev, bW, alpha, x, num_groups, out=None):
+    N, K, nb = bW.shape[2], bW.shape[0] * 32, bW.shape[1]
+    M = x.shape[0]
+    d_out = (torch.zeros((M, N), dtype=torch.float16) if out is None else out.clone()).to(dev)
+    d_bW, d_a, d_x = bW.to(dev), alpha.to(dev), x.to(dev).contiguous()
+    _check(native.cabi().lutgemm_gemv_rowwise_f16(_ptr(d_bW), _ptr(d_a), _ptr(d_x), _ptr(d_out),
+                                                  N, K, nb, num_groups, M, _stream()))
+    torch.cuda.synchronize()
+    return d_out
+
+
+def run_block(dev, bW, alpha, x, R, kind, out=None):
+    N, K, nb = bW.shape[2], bW.shape[0] * 32, bW.shape[1]
+    M = x.shape[0]
+    d_out = (torch.zeros((M, N), dtype=torch.float16) if out is None else out.clone()).to(dev)
+    d_bW, d_a, d_x = bW.to(dev), alpha.to(dev), x.to(dev).contiguous()
+    lib = native.cabi()
+    if kind == orc.ALPHA_F16:
+        rc = lib.lutgemm_gemv_block_f16(_ptr(d_bW), _ptr(d_a), _ptr(d_x), _ptr(d_out), N, K, nb, R, M, _stream())
+    elif kind == orc.ALPHA_SHIFT_U16:
+        rc = lib.lutgemm_gemv_block_shift_u16(_ptr(d_bW), _ptr(d_a), _ptr(d_x), _ptr(d_out), N, K, nb, R, 3, M,
+                                              _stream())
+    else:
+        rc = lib.lutgemm_gemv_block_apot_i8(_ptr(d_bW), _ptr(d_a), _ptr(d_x), _ptr(d_out), N, K, nb, R, 3, M,
+                                            _stream())
+    _check(rc)
+    torch.cuda.synchronize()
+    return d_out
+
+
+# ---- row-wise alpha (configs 1, 2, 4, 5) -------------------------------------
+
+def test_config1_opt125m_fc1_real_bcq(gpu_device):
+    N, K = workload.OPT125M_FC1
+    p = workload.make_rowwise_problem(N, K, nb=3, group_size=128, seed=0)
+    # operands are bit-exact restatements of the reference packing
+    assert np.array_equal(p.bW.permute(2, 0, 1).contiguous().numpy(),
+                          orc.pack_binary_weight_c(p.B.numpy()))
+    want, y32 = orc.gemv_rowwise_c(p.bW.numpy(), p.alpha.numpy(), p.x.numpy(), p.num_groups)
+    got = run_rowwise(gpu_device, p.bW, p.alpha, p.x, p.num_groups)
+    _assert_close(got, want, "config1")
+    # and against the dense dequantise-and-matmul path
+    Wq = orc.dequant_rowwise_kernel_layout(p.bW.numpy(), p.alpha.numpy())
+    _assert_close(got, orc.dense_gemv_np(Wq, p.x.numpy()), "config1 dense")
+
+
+@pytest.mark.parametrize("N,K,nb,gs,M", [
+    (4, 32, 1, 32, 1),         # smallest legal problem
+    (8, 64, 2, 32, 1),
+    (132, 96, 3, 96, 1),       # N tail inside a step, K not a multiple of 256
+    (260, 288, 4, 32, 2),      # partial table set, two rows
+    (512, 512, 3, 128, 1),
+    (1024, 768, 2, 256, 3),
+    (3072, 768, 3, 128, 5),    # config-1 shape with a batch
+    (384, 2048, 4, 2048, 1),   # a single group along K
+    (128, 8192, 3, 128, 1),    # long K, one N tile
+])
+def test_rowwise_ragged_shapes(gpu_device, N, K, nb, gs, M):
+    p = workload.make_rowwise_problem(N, K, nb=nb, group_size=gs, M=M, seed=N + K + nb, quantize=False)
+    want, _ = orc.gemv_rowwise_c(p.bW.numpy(), p.alpha.numpy(), p.x.numpy(), p.num_groups)
+    got = run_rowwise(gpu_device, p.bW, p.alpha, p.x, p.num_groups)
+    _assert_close(got, want, (N, K, nb, gs, M))
+
+
+def test_rowwise_general_alpha_values(gpu_device):
+    # the binding accepts any fp16 alpha, not only powers of two
+    g = torch.Generator().manual_seed(5)
+    N, K, nb, gs = 256, 512, 3, 64
+    p = workload.make_rowwise_problem(N, K, nb=nb, group_size=gs, seed=5, quantize=False)
+    alpha = (torch.rand(p.alpha.shape, generator=g) * 0.05).half()
+    want, _ = orc.gemv_rowwise_c(p.bW.numpy(), alpha.numpy(), p.x.numpy(), p.num_groups)
+    _assert_close(run_rowwise(gpu_device, p.bW, alpha, p.x, p.num_groups), want)
+
+
+def test_accumulates_into_bias_and_is_deterministic(gpu_device):
+    N, K = 1024, 1024
+    p = workload.make_rowwise_problem(N, K, nb=3, group_size=128, M=2, seed=9, quantize=False)
+    bias = (torch.randn((2, N), generator=torch.Generator().manual_seed(1))).half()
+    want, _ = orc.gemv_rowwise_c(p.bW.numpy(), p.alpha.numpy(), p.x.numpy(), p.num_groups, out=bias.numpy())
+    got1 = run_rowwise(gpu_device, p.bW, p.alpha, p.x, p.num_groups, out=bias)
+    got2 = run_rowwise(gpu_device, p.bW, p.alpha, p.x, p.num_groups, out=bias)
+    _assert_close(got1, want)
+    assert torch.equal(got1, got2)                      # fixed summation order
+    # x = 0 leaves the pre-filled output untouched, bit for bit
+    zero = torch.zeros_like(p.x)
+    assert torch.equal(run_rowwise(gpu_device, p.bW, p.alpha, zero, p.num_groups, out=bias).cpu(), bias)
+
+
+def test_unit_vectors_return_columns_of_wq(gpu_device):
+    N, K, nb, gs = 256, 512, 3, 128
+    p = workload.make_rowwise_problem(N, K, nb=nb, group_size=gs, seed=3, quantize=False)
+    Wq = orc.dequant_rowwise_kernel_layout(p.bW.numpy(), p.alpha.numpy())
+    ks = [0, 7, 8, 31, 32, 255, 256, 511]
+    x = torch.zeros((len(ks), K), dtype=torch.float16)
+    for i, k in enumerate(ks):
+        x[i, k] = 1.0
+    got = run_rowwise(gpu_device, p.bW, p.alpha, x, p.num_groups).float().cpu().numpy()
+    for i, k in enumerate(ks):
+        # W_q entries are sums of <= 3 powers of two: exactly representable in fp16 here
+        assert np.array_equal(got[i], Wq[:, k].astype(np.float16).astype(np.float32)), k
+
+
+@pytest.mark.parametrize("name,N,K", workload.LLAMA2_7B_LINEARS[3:])   # o_proj, gate, up, down
+def test_config2_llama7b_shapes_real_bcq(gpu_device, name, N, K):
+    # quantise on the GPU (pure torch), check against the CPU oracle at full size
+    p = workload.make_rowwise_problem(N, K, nb=3, group_size=128, seed=0, device=gpu_device)
+    bW, alpha, x = p.bW.cpu(), p.alpha.cpu(), p.x.cpu()
+    want, _ = orc.gemv_rowwise_c(bW.numpy(), alpha.numpy(), x.numpy(), p.num_groups)
+    got = run_rowwise(gpu_device, bW, alpha, x, p.num_groups)
+    _assert_close(got, want, name)
+    # linearity, a size-independent property: f(x1) + f(x2) == f(x1 + x2) up to fp16 rounding
+    x2 = torch.randn((1, K), generator=torch.Generator().manual_seed(4)).half()
+    y1 = got.float()
+    y2 = run_rowwise(gpu_device, bW, alpha, x2, p.num_groups).float()
+    y12 = run_rowwise(gpu_device, bW, alpha, (x.float() + x2.float()).half(), p.num_groups).float()
+    rel, _ = orc.error_metrics((y1 + y2).cpu().numpy(), y12.cpu().numpy())
+    assert rel < 3e-3
+
+
+@pytest.mark.parametrize("N,K,nb", [(8192, 8192, 2), (1024, 8192, 4), (8192, 8192, 4)])
+def test_config5_llama70b_shapes_m1(gpu_device, N, K, nb):
+    p = workload.make_rowwise_problem(N, K, nb=nb, group_size=128, seed=1, sigma=0.015, quantize=False)
+    want, _ = orc.gemv_rowwise_c(p.bW.numpy(), p.alpha.numpy(), p.x.numpy(), p.num_groups)
+    _assert_close(run_rowwise(gpu_device, p.bW, p.alpha, p.x, p.num_groups), want)
+
+
+@pytest.mark.parametrize("M", [4, 16, 32])
+def test_config5_small_batches(gpu_device, M):
+    N, K, nb = 1024, 8192, 2
+    p = workload.make_rowwise_problem(N, K, nb=nb, group_size=128, M=M, seed=2, sigma=0.015, quantize=False)
+    want, _ = orc.gemv_rowwise_c(p.bW.numpy(), p.alpha.numpy(), p.x.numpy(), p.num_groups)
+    _assert_close(run_rowwise(gpu_device, p.bW, p.alpha, p.x, p.num_groups), want)
+
+
+# ---- block alpha (config 3 and the LutLinear default format) -----------------
+
+def test_config3_llama13b_block_real_bcq(gpu_device):
+    N, K = workload.LLAMA2_13B_SHAPES[0]
+    p = workload.make_block_problem(N, K, nb=2, R=8, seed=0, device=gpu_device)
+    bW, alpha, x = p.bW.cpu(), p.alpha.cpu(), p.x.cpu()
+    want, _ = orc.gemv_block_c(bW.numpy(), alpha.numpy(), x.numpy(), 8, kind=orc.ALPHA_F16)
+    _assert_close(run_block(gpu_device, bW, alpha, x, 8, orc.ALPHA_F16), want)
+    # dense path from the ON-DISK tensors (dequantise, transpose, matmul)
+    W = orc.dequant_lat_disk(p.disk_bWeight.cpu().numpy(), p.disk_alpha.cpu().numpy())
+    _assert_close(run_block(gpu_device, bW, alpha, x, 8, orc.ALPHA_F16), orc.dense_gemv_np(W, x.numpy()))
+
+
+@pytest.mark.parametrize("N,K", workload.LLAMA2_13B_SHAPES[1:])
+def test_config3_non_square_shapes(gpu_device, N, K):
+    p = workload.make_block_problem(N, K, nb=2, R=8, seed=1, quantize=False)
+    want, _ = orc.gemv_block_c(p.bW.numpy(), p.alpha.numpy(), p.x.numpy(), 8, kind=orc.ALPHA_F16)
+    _assert_close(run_block(gpu_device, p.bW, p.alpha, p.x, 8, orc.ALPHA_F16), want)
+
+
+@pytest.mark.parametrize("N,K,nb,R,M", [(32, 32, 1, 1, 1), (64, 96, 3, 4, 2), (640, 288, 2, 8, 1),
+                                         (256, 512, 4, 64, 3), (1024, 1024, 3, 8, 1)])
+def test_block_f16_ragged(gpu_device, N, K, nb, R, M):
+    p = workload.make_block_problem(N, K, nb=nb, R=R, M=M, seed=N + R, quantize=False)
+    want, _ = orc.gemv_block_c(p.bW.numpy(), p.alpha.numpy(), p.x.numpy(), R, kind=orc.ALPHA_F16)
+    _assert_close(run_block(gpu_device, p.bW, p.alpha, p.x, R, orc.ALPHA_F16), want)
+
+
+@pytest.mark.parametrize("N,K,nb,R,M", [(64, 64, 2, 8, 1), (768, 768, 3, 8, 1), (512, 1024, 3, 16, 2)])
+def test_block_shift_u16(gpu_device, N, K, nb, R, M):
+    p = workload.make_block_problem(N, K, nb=nb, R=R, M=M, seed=3, quantize=False)
+    g = torch.Generator().manual_seed(N)
+    code = torch.randint(0, 512, (K // 8, nb, R), generator=g).to(torch.int16)
+    x = (p.x.float() * 0.01).half()          # multipliers reach 384: keep outputs inside fp16
+    want, _ = orc.gemv_block_c(p.bW.numpy(), code.numpy(), x.numpy(), R, kind=orc.ALPHA_SHIFT_U16)
+    _assert_close(run_block(gpu_device, p.bW, code, x, R, orc.ALPHA_SHIFT_U16), want)
+
+
+@pytest.mark.parametrize("N,K,nb,R,M", [(64, 64, 2, 8, 1), (768, 768, 3, 8, 1), (3072, 768, 3, 8, 1),
+                                         (512, 1024, 3, 16, 2)])
+def test_block_apot_i8(gpu_device, N, K, nb, R, M):
+    p = workload.make_block_problem(N, K, nb=nb, R=R, M=M, seed=4, quantize=False)
+    g = torch.Generator().manual_seed(K)
+    code = torch.randint(-12, -3, (K // 8, nb, R, 3), generator=g).to(torch.int8)
+    code[torch.rand(code.shape, generator=g) < 0.4] = -128       # absent terms
+    want, _ = orc.gemv_block_c(p.bW.numpy(), code.numpy(), p.x.numpy(), R, kind=orc.ALPHA_APOT_I8)
+    _assert_close(run_block(gpu_device, p.bW, code, p.x, R, orc.ALPHA_APOT_I8), want)
+
+
+# ---- uniform mode -------------------------------------------------------------
+
+@pytest.mark.parametrize("N,K,nb,gs,M", [(64, 128, 3, 64, 1), (1024, 1024, 4, 128, 1), (260, 288, 2, 32, 2)])
+def test_uniform_mode(gpu_device, N, K, nb, gs, M):
+    p = workload.make_rowwise_problem(N, K, nb=nb, group_size=gs, M=M, seed=6, quantize=False)
+    g = torch.Generator().manual_seed(7)
+    alpha = (torch.rand((K // gs, N), generator=g) * 0.05).half()
+    q = (torch.randn((K // gs, N), generator=g) * 0.01).half()
+    want, _ = orc.gemv_uniform_c(p.bW.numpy(), alpha.numpy(), q.numpy(), p.x.numpy(), K // gs)
+    dev = gpu_device
+    d_out = torch.zeros((M, N), dtype=torch.float16, device=dev)
+    d = [t.to(dev) for t in (p.bW, alpha, q, p.x)]
+    _check(native.cabi().lutgemm_gemv_uniform_f16(_ptr(d[0]), _ptr(d[1]), _ptr(d[2]), _ptr(d[3]), _ptr(d_out),
+                                                  N, K, nb, K // gs, M, _stream()))
+    torch.cuda.synchronize()
+    _assert_close(d_out, want)
+
+
+# ---- the Python operator surface ----------------------------------------------
+
+def test_python_module_and_lutlinear(gpu_device):
+    from shiftaddllm_amd.lut_gemm.quant import LutLinear, encode_apot_int8
+    dev = gpu_device
+    ext = native.lutgemm
+    N, K, R, nb = 768, 768, 8, 3
+    p = workload.make_block_problem(N, K, nb=nb, R=R, seed=0)
+    bias = (torch.randn(N, generator=torch.Generator().manual_seed(2)) * 0.1).half()
+
+    # reference call pattern: output = bias.clone(); ext(output, ...) (lut_gemm/quant.py:46-51)
+    code = encode_apot_int8(p.alpha.float())                      # exact: alphas are powers of two
+    out = bias.clone().to(dev).reshape(1, N)
+    ext.lutgemm_compute_block_shiftInt8(out, p.bW.to(dev), code.to(dev), p.x.to(dev), N, K, nb, R, 3)
+    torch.cuda.synchronize()
+    want, _ = orc.gemv_block_c(p.bW.numpy(), p.alpha.numpy(), p.x.numpy(), R, kind=orc.ALPHA_F16,
+                               out=bias.numpy().reshape(1, N))
+    _assert_close(out, want)
+
+    lin = LutLinear(K, N, group_size=K // R, wbit=nb, bias=bias.to(dev)).to(dev)
+    lin.binaryWeight.data = p.bW.to(dev)
+    lin.alpha.data = lin.quantize_to_apot(p.alpha.float()).to(dev)
+    y = lin(p.x.to(dev).reshape(1, 1, K))                          # [batch, token, K] like a decoder
+    assert tuple(y.shape) == (1, 1, N) and y.dtype == torch.float16
+    _assert_close(y.reshape(1, N), want)
+
+    # no bias (Llama) and several tokens: supersets of the reference behaviour
+    lin2 = LutLinear(K, N, group_size=K // R, wbit=nb, bias=None, alpha_format="block_fp16").to(dev)
+    lin2.binaryWeight.data = p.bW.to(dev)
+    lin2.alpha.data = p.alpha.to(dev)
+    x4 = torch.randn((2, 2, K), generator=torch.Generator().manual_seed(3)).half()
+    y4 = lin2(x4.to(dev))
+    want4, _ = orc.gemv_block_c(p.bW.numpy(), p.alpha.numpy(), x4.reshape(4, K).numpy(), R, kind=orc.ALPHA_F16)
+    assert tuple(y4.shape) == (2, 2, N)
+    _assert_close(y4.reshape(4, N), want4)
+
+    # wrong dtype / shape raise instead of corrupting memory
+    with pytest.raises(RuntimeError):
+        ext.lutgemm_compute_block(out, p.bW.to(dev), p.alpha.float().to(dev), p.x.to(dev), N, K, nb, R)
+    with pytest.raises(RuntimeError):
+        ext.lutgemm_compute_block(out, p.bW.to(dev)[:, :, :-4].contiguous(), p.alpha.to(dev), p.x.to(dev),
+                                  N, K, nb, R)
+    with pytest.raises(RuntimeError):
+        ext.lutgemm_compute_block_shiftInt8(out, p.bW.to(dev), code.to(dev), p.x.to(dev), N, K, nb, R, 2)
+
+
+def test_runs_on_a_side_stream(gpu_device):
+    p = workload.make_rowwise_problem(512, 1024, nb=3, group_size=128, seed=8, quantize=False)
+    want, _ = orc.gemv_rowwise_c(p.bW.numpy(), p.alpha.numpy(), p.x.numpy(), p.num_groups)
+    s = torch.cuda.Stream()
+    with torch.cuda.stream(s):
+        got = run_rowwise(gpu_device, p.bW, p.alpha, p.x, p.num_groups)
+    s.synchronize()
+    _assert_close(got, want)
