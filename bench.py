@@ -1,0 +1,303 @@
+#!/usr/bin/env python3
+"""Benchmark of the LUT-GEMM hot path on one MI355X.
+
+Workload (BASELINE.json configs[1]): the seven linear layers of a Llama-2-7B
+decoder block as 3-bit BCQ LUT-GEMVs (group 128 along K, power-of-two alphas,
+batch 1).  One *step* is one decoded token's worth of them: 32 blocks x 7
+GEMVs = 224 launches streaming 2.74 GB of distinct weights (so nothing is
+served from the 256 MB Infinity Cache), replayed from one HIP graph.
+
+Prints ONE JSON line.  `value` is the mean device time per GEMV call in that
+sequence, in microseconds, with all operands resident in HBM.  `roofline`
+prices the same launches against the 8 TB/s HBM peak using the algorithmic
+bytes per call (signs + alphas + x + y read + y write).  `cpu_baseline` is the
+reference's CPU-executable path (dequantise once, fp32 linear) timed on this
+box's host cores on one decoder block.
+
+Run with no arguments for the default configuration; `--gpus` above 1 is
+refused (this build is single-GPU).
+"""
+from __future__ import annotations
+
+import argparse
+import ctypes
+import json
+import os
+import statistics
+import sys
+import time
+
+REPO = os.path.dirname(os.path.abspath(__file__))
+if REPO not in sys.path:
+    sys.path.insert(0, REPO)
+
+HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
+N_LAYERS = 32
+NB, GROUP = 3, 128
+TRAFFIC_NOTE = os.path.join(REPO, "profiles", "lut_gemv_llama7b_3bit_pmc.md")
+
+
+def parse_args():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--layers", type=int, default=N_LAYERS, help="distinct decoder blocks in the weight pool")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying a HIP graph")
+    ap.add_argument("--shape-table", action="store_true", help="also time every shape alone, hot and rotating")
+    ap.add_argument("--profile-shape", type=str, default="",
+                    help="N,K[,nb[,iters]]: only launch this shape repeatedly (for rocprofv3 runs) and exit")
+    ap.add_argument("--profile-copy", type=int, default=0,
+                    help="bytes: only run the calibration copy kernel a few times (for rocprofv3 --pmc) and exit")
+    return ap.parse_args()
+
+
+class Gemv:
+    """Device operands of one row-wise-alpha LUT-GEMV."""
+
+    def __init__(self, torch, dev, N, K, nb, seed, x=None):
+        g = torch.Generator(device=dev).manual_seed(seed)
+        self.N, self.K, self.nb = N, K, nb
+        self.groups = K // GROUP
+        self.bW = torch.randint(-2 ** 31, 2 ** 31 - 1, (K // 32, nb, N), generator=g, device=dev,
+                                dtype=torch.int32)
+        # power-of-two scales shaped like BCQ output: per (group, row) a base exponent, halving per bit plane
+        e = torch.randint(-9, -5, (self.groups, 1, N), generator=g, device=dev).float()
+        e = e - torch.arange(nb, device=dev).float().view(1, nb, 1)
+        self.alpha = torch.exp2(e).to(torch.float16).contiguous()
+        self.x = x if x is not None else torch.randn((1, K), generator=g, device=dev).half()
+        self.out = torch.zeros((1, N), dtype=torch.float16, device=dev)
+        self.bytes = None
+
+    def args(self):
+        p = lambda t: ctypes.c_void_p(t.data_ptr())
+        return (p(self.bW), p(self.alpha), p(self.x), p(self.out), self.N, self.K, self.nb, self.groups, 1)
+
+
+def main():
+    args = parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on ONE GPU (no sharding, no collectives); "
+              f"--gpus {args.gpus} is not supported.", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    from shiftaddllm_amd import native, workload
+
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        sys.exit(1)
+    dev = torch.device("cuda:0")
+    lib = native.cabi()            # raises if the HIP library is not built: no fallback
+    launch = lib.lutgemm_gemv_rowwise_f16
+
+    def run(g, stream_ptr):
+        rc = launch(*g.args(), stream_ptr)
+        if rc:
+            raise RuntimeError(lib.lutgemm_strerror(rc).decode())
+
+    def alg_bytes(g):
+        return lib.lutgemm_algorithmic_bytes(g.N, g.K, g.nb, 1, g.groups * g.nb * g.N, 2)
+
+    stream = torch.cuda.Stream()
+    sp = ctypes.c_void_p(stream.cuda_stream)
+
+    # ---- profiler helper modes --------------------------------------------
+    if args.profile_copy:
+        nbytes = args.profile_copy // 16 * 16
+        src = torch.empty(nbytes, dtype=torch.uint8, device=dev).random_(0, 255)
+        dst = torch.empty_like(src)
+        with torch.cuda.stream(stream):
+            for _ in range(5):
+                lib.lutgemm_copy_bytes(ctypes.c_void_p(dst.data_ptr()), ctypes.c_void_p(src.data_ptr()), nbytes, sp)
+        stream.synchronize()
+        print(json.dumps({"copy_bytes": nbytes, "launches": 5}))
+        return
+    if args.profile_shape:
+        parts = [int(v) for v in args.profile_shape.split(",")]
+        N, K = parts[0], parts[1]
+        nb = parts[2] if len(parts) > 2 else NB
+        iters = parts[3] if len(parts) > 3 else 8
+        pool = [Gemv(torch, dev, N, K, nb, 100 + i) for i in range(iters)]
+        with torch.cuda.stream(stream):
+            for g in pool:      # each launch touches weights never read before
+                run(g, sp)
+        stream.synchronize()
+        print(json.dumps({"shape": [N, K, nb], "launches": iters, "algorithmic_bytes_per_launch": alg_bytes(pool[0])}))
+        return
+
+    # ---- weight pool: `layers` decoder blocks x 7 linears -----------------
+    t0 = time.time()
+    pool = []
+    for layer in range(args.layers):
+        x_hidden = torch.randn((1, 4096), generator=torch.Generator(device=dev).manual_seed(7 + layer),
+                               device=dev).half()
+        x_inter = torch.randn((1, 11008), generator=torch.Generator(device=dev).manual_seed(9 + layer),
+                              device=dev).half()
+        for j, (name, N, K) in enumerate(workload.LLAMA2_7B_LINEARS):
+            pool.append(Gemv(torch, dev, N, K, NB, 1000 * layer + j, x=x_hidden if K == 4096 else x_inter))
+    for g in pool:
+        g.bytes = alg_bytes(g)
+    step_bytes = sum(g.bytes for g in pool)
+    calls_per_step = len(pool)
+    torch.cuda.synchronize()
+    t_pool = time.time() - t0
+
+    # ---- parity spot check against the CPU oracle (checker only) ----------
+    import numpy as np
+    import oracle
+    parity = {}
+    for g in pool[3:7]:                       # o_proj, gate, up, down of block 0
+        g.out.zero_()
+        with torch.cuda.stream(stream):
+            run(g, sp)
+        stream.synchronize()
+        want, _ = oracle.gemv_rowwise_c(g.bW.cpu().numpy(), g.alpha.cpu().numpy(), g.x.cpu().numpy(), g.groups)
+        rel, mad = oracle.error_metrics(g.out.float().cpu().numpy(), want.astype(np.float32))
+        parity[f"{g.N}x{g.K}"] = {"rel_l2": rel, "max_rel": mad}
+        if rel > 2e-3 or mad > 1e-2:
+            raise SystemExit(f"parity failure on {g.N}x{g.K}: rel_l2={rel} max={mad}")
+
+    # ---- the timed step -----------------------------------------------------
+    def one_step_eager():
+        for g in pool:
+            run(g, sp)
+
+    with torch.cuda.stream(stream):
+        one_step_eager()                      # sizes the workspace of this stream before any capture
+    stream.synchronize()
+
+    graph = None
+    if not args.no_graph:
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=stream):
+            one_step_eager()
+
+    def step():
+        if graph is not None:
+            graph.replay()
+        else:
+            with torch.cuda.stream(stream):
+                one_step_eager()
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t_start = time.perf_counter()
+    with torch.cuda.stream(stream):
+        ev0.record(stream)
+    for _ in range(args.steps):
+        step()
+    with torch.cuda.stream(stream):
+        ev1.record(stream)
+    torch.cuda.synchronize()
+    wall_s = time.perf_counter() - t_start
+    dev_ms = ev0.elapsed_time(ev1)            # HIP events on the launch stream
+
+    ms_per_step = wall_s * 1e3 / args.steps
+    dev_ms_per_step = dev_ms / args.steps
+    us_per_call = dev_ms_per_step * 1e3 / calls_per_step
+    achieved_gbs = step_bytes / (dev_ms_per_step * 1e-3) / 1e9
+
+    # ---- optional per-shape table -------------------------------------------
+    shape_table = None
+    if args.shape_table:
+        shape_table = {}
+        for (N, K) in ((4096, 4096), (11008, 4096), (4096, 11008)):
+            same = [g for g in pool if (g.N, g.K) == (N, K)]
+            row = {}
+            for label, seq in (("hot", [same[0]] * 64), ("rotating", (same * 8)[:max(64, len(same))])):
+                with torch.cuda.stream(stream):
+                    for g in seq[:4]:
+                        run(g, sp)
+                stream.synchronize()
+                gr = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(gr, stream=stream):
+                    for g in seq:
+                        run(g, sp)
+                times = []
+                for _ in range(7):
+                    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                    with torch.cuda.stream(stream):
+                        a.record(stream)
+                    gr.replay()
+                    with torch.cuda.stream(stream):
+                        b.record(stream)
+                    torch.cuda.synchronize()
+                    times.append(a.elapsed_time(b) * 1e3 / len(seq))
+                us = statistics.median(times)
+                row[label] = {"us_per_call": round(us, 3), "GBps": round(same[0].bytes / us / 1e3, 1),
+                              "frac_hbm_peak": round(same[0].bytes / us / 1e3 / HBM_PEAK_GBS, 4)}
+            row["algorithmic_bytes"] = same[0].bytes
+            shape_table[f"{N}x{K}"] = row
+
+    # ---- CPU baseline: dequantise once + fp32 linear on host cores ----------
+    cpu = None
+    if not args.no_cpu_baseline:
+        threads = torch.get_num_threads()
+        block = pool[:7]
+        runs = []
+        for g in block:
+            f, _ = oracle.cpu_dense_path(g.bW.cpu().numpy(), g.alpha.cpu().numpy())
+            runs.append((f, g.x.cpu()))
+        for f, x in runs:
+            f(x)
+        samples = []
+        t_lim = time.time() + 20.0
+        while len(samples) < 10 and time.time() < t_lim:
+            t = time.perf_counter()
+            for f, x in runs:
+                f(x)
+            samples.append((time.perf_counter() - t) / len(runs))
+        cpu = {"value": round(statistics.median(samples) * 1e6, 1), "unit": "us/call", "cores": threads,
+               "kind": "port",
+               "sample": f"one decoder block (7 GEMVs of this workload), weights dequantised once, fp32 "
+                         f"torch linear, median of {len(samples)} passes; host shows {os.cpu_count()} cpus"}
+
+    traffic = None
+    if os.path.exists(TRAFFIC_NOTE):
+        for line in open(TRAFFIC_NOTE):
+            if line.startswith("traffic_bytes_per_launch:"):
+                traffic = float(line.split(":", 1)[1].strip())
+
+    mean_bytes = step_bytes / calls_per_step
+    result = {
+        "metric": "lut_gemv_us_per_call_llama2_7b_3bit_batch1",
+        "value": round(us_per_call, 4),
+        "unit": "us/call",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 5),
+        "higher_is_better": False,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": "llama2-7b linears, 3-bit BCQ, group 128, pow2 alpha, batch 1: "
+                               f"{args.layers} blocks x 7 GEMVs per step over distinct weights "
+                               f"({step_bytes / 1e9:.3f} GB/step)",
+                   "launch": "eager" if graph is None else "hip-graph replay",
+                   "calls_per_step": calls_per_step},
+        "device_ms_per_step": round(dev_ms_per_step, 5),
+        "achieved_GBps": round(achieved_gbs, 1),
+        "frac_hbm_peak": round(achieved_gbs / HBM_PEAK_GBS, 4),
+        "decode_tokens_per_s_linears_only": round(1e3 / dev_ms_per_step, 1),
+        "roofline": {"bound": "hbm", "achieved": round(achieved_gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(achieved_gbs / HBM_PEAK_GBS, 4), "traffic": traffic,
+                     "kernel": "lut_gemv_kernel<3,2,row-wise>",
+                     "algorithmic_bytes_per_launch": round(mean_bytes),
+                     "avg_launch_us": round(us_per_call, 4)},
+        "cpu_baseline": cpu,
+        "parity": parity,
+        "pool_build_s": round(t_pool, 2),
+    }
+    if shape_table is not None:
+        result["shapes"] = shape_table
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

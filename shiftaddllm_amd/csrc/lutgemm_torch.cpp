@@ -11,8 +11,8 @@
 //  * `d_input` may hold M rows ([M, K] or [..., K]); the reference's row-wise
 //    and uniform entry points are batch-1 only.
 #include <torch/extension.h>
-#include <c10/hip/HIPGuard.h>
-#include <c10/hip/HIPStream.h>
+#include <ATen/hip/impl/HIPGuardImplMasqueradingAsCUDA.h>
+#include <ATen/hip/impl/HIPStreamMasqueradingAsCUDA.h>
 
 #include <string>
 
@@ -78,11 +78,11 @@ void lutgemm_compute_shift_scale(torch::Tensor output, torch::Tensor bWeight, to
     TORCH_CHECK(num_groups > 0 && kSize % num_groups == 0 && (kSize / num_groups) % 32 == 0,
                 "kSize/num_groups must be a multiple of 32");
     check_alpha(alpha, output, torch::kHalf, num_groups * nb * mSize, "alpha [num_groups, nb, mSize]");
-    const c10::hip::HIPGuard guard(output.device());
+    const c10::hip::HIPGuardMasqueradingAsCUDA guard(output.device());
     int rc = lutgemm_gemv_rowwise_f16((const uint32_t *)bWeight.data_ptr<int32_t>(), alpha.data_ptr(),
                                       d_input.data_ptr(), output.data_ptr(), (int)mSize, (int)kSize,
                                       (int)nb, (int)num_groups, rows_of(d_input, kSize),
-                                      c10::hip::getCurrentHIPStream().stream());
+                                      c10::hip::getCurrentHIPStreamMasqueradingAsCUDA().stream());
     raise_on_error(rc, "lutgemm_compute_shift_scale");
 }
 
@@ -96,12 +96,12 @@ void lutgemm_compute(torch::Tensor output, torch::Tensor bWeight, torch::Tensor 
                 "kSize/num_groups must be a multiple of 32");
     check_alpha(alpha, output, torch::kHalf, num_groups * mSize, "alpha [num_groups, mSize]");
     check_alpha(q_bias, output, torch::kHalf, num_groups * mSize, "q_bias [num_groups, mSize]");
-    const c10::hip::HIPGuard guard(output.device());
+    const c10::hip::HIPGuardMasqueradingAsCUDA guard(output.device());
     int rc = lutgemm_gemv_uniform_f16((const uint32_t *)bWeight.data_ptr<int32_t>(), alpha.data_ptr(),
                                       q_bias.data_ptr(), d_input.data_ptr(), output.data_ptr(),
                                       (int)mSize, (int)kSize, (int)nb, (int)num_groups,
                                       rows_of(d_input, kSize),
-                                      c10::hip::getCurrentHIPStream().stream());
+                                      c10::hip::getCurrentHIPStreamMasqueradingAsCUDA().stream());
     raise_on_error(rc, "lutgemm_compute");
 }
 
@@ -120,11 +120,11 @@ void lutgemm_compute_block(torch::Tensor output, torch::Tensor bWeight, torch::T
     check_block(mSize, num_groups);
     check_alpha(alpha, output, torch::kHalf, (kSize / 8) * nb * num_groups,
                 "alpha [kSize/8, nb, num_groups]");
-    const c10::hip::HIPGuard guard(output.device());
+    const c10::hip::HIPGuardMasqueradingAsCUDA guard(output.device());
     int rc = lutgemm_gemv_block_f16((const uint32_t *)bWeight.data_ptr<int32_t>(), alpha.data_ptr(),
                                     d_input.data_ptr(), output.data_ptr(), (int)mSize, (int)kSize,
                                     (int)nb, (int)num_groups, rows_of(d_input, kSize),
-                                    c10::hip::getCurrentHIPStream().stream());
+                                    c10::hip::getCurrentHIPStreamMasqueradingAsCUDA().stream());
     raise_on_error(rc, "lutgemm_compute_block");
 }
 
@@ -138,13 +138,13 @@ void lutgemm_compute_block_shift(torch::Tensor output, torch::Tensor bWeight, to
     TORCH_CHECK(num_apot == 3, "num_apot must be 3 (the packed uint16 always carries three shift fields)");
     check_alpha(alpha, output, torch::kShort, (kSize / 8) * nb * num_groups,
                 "alpha [kSize/8, nb, num_groups] (int16 holding uint16 shift fields)");
-    const c10::hip::HIPGuard guard(output.device());
+    const c10::hip::HIPGuardMasqueradingAsCUDA guard(output.device());
     int rc = lutgemm_gemv_block_shift_u16((const uint32_t *)bWeight.data_ptr<int32_t>(),
                                           (const uint16_t *)alpha.data_ptr<int16_t>(),
                                           d_input.data_ptr(), output.data_ptr(), (int)mSize,
                                           (int)kSize, (int)nb, (int)num_groups, (int)num_apot,
                                           rows_of(d_input, kSize),
-                                          c10::hip::getCurrentHIPStream().stream());
+                                          c10::hip::getCurrentHIPStreamMasqueradingAsCUDA().stream());
     raise_on_error(rc, "lutgemm_compute_block_shift");
 }
 
@@ -158,12 +158,12 @@ void lutgemm_compute_block_shiftInt8(torch::Tensor output, torch::Tensor bWeight
     TORCH_CHECK(num_apot == 3, "num_apot must be 3 (alpha carries three int8 exponents per entry)");
     check_alpha(alpha, output, torch::kChar, (kSize / 8) * nb * num_groups * 3,
                 "alpha [kSize/8, nb, num_groups, 3]");
-    const c10::hip::HIPGuard guard(output.device());
+    const c10::hip::HIPGuardMasqueradingAsCUDA guard(output.device());
     int rc = lutgemm_gemv_block_apot_i8((const uint32_t *)bWeight.data_ptr<int32_t>(),
                                         alpha.data_ptr<int8_t>(), d_input.data_ptr(),
                                         output.data_ptr(), (int)mSize, (int)kSize, (int)nb,
                                         (int)num_groups, (int)num_apot, rows_of(d_input, kSize),
-                                        c10::hip::getCurrentHIPStream().stream());
+                                        c10::hip::getCurrentHIPStreamMasqueradingAsCUDA().stream());
     raise_on_error(rc, "lutgemm_compute_block_shiftInt8");
 }
 
@@ -173,9 +173,9 @@ void copy_bytes(torch::Tensor dst, torch::Tensor src)
     TORCH_CHECK(dst.is_cuda() && src.is_cuda() && dst.is_contiguous() && src.is_contiguous(),
                 "copy_bytes needs contiguous GPU tensors");
     TORCH_CHECK(dst.nbytes() == src.nbytes() && dst.nbytes() % 16 == 0, "sizes must match, multiple of 16");
-    const c10::hip::HIPGuard guard(dst.device());
+    const c10::hip::HIPGuardMasqueradingAsCUDA guard(dst.device());
     int rc = lutgemm_copy_bytes(dst.data_ptr(), src.data_ptr(), dst.nbytes(),
-                                c10::hip::getCurrentHIPStream().stream());
+                                c10::hip::getCurrentHIPStreamMasqueradingAsCUDA().stream());
     raise_on_error(rc, "copy_bytes");
 }
 

@@ -34,9 +34,12 @@ def _check(rc):
     assert rc == 0, native.cabi().lutgemm_strerror(rc).decode()
 
 
-def _assert_close(y_gpu, y_ref, what=""):
+def _assert_close(y_gpu, y_ref, what="", margin=TIGHT):
+    """y_ref is the oracle's fp16 output (same single rounding as the kernel):
+    held to a tenth of the bars.  Against an un-rounded fp32 reference pass
+    margin=0.25, fp16 rounding alone costs about 2e-4."""
     rel, mad = orc.error_metrics(y_gpu.float().cpu().numpy(), np.asarray(y_ref, dtype=np.float32))
-    assert rel <= REL_L2_BAR * TIGHT and mad <= MAX_ABS_BAR * TIGHT, (what, rel, mad)
+    assert rel <= REL_L2_BAR * margin and mad <= MAX_ABS_BAR * margin, (what, rel, mad)
     return rel, mad
 
 
@@ -83,7 +86,7 @@ def test_config1_opt125m_fc1_real_bcq(gpu_device):
     _assert_close(got, want, "config1")
     # and against the dense dequantise-and-matmul path
     Wq = orc.dequant_rowwise_kernel_layout(p.bW.numpy(), p.alpha.numpy())
-    _assert_close(got, orc.dense_gemv_np(Wq, p.x.numpy()), "config1 dense")
+    _assert_close(got, orc.dense_gemv_np(Wq, p.x.numpy()), "config1 dense", margin=0.25)
 
 
 @pytest.mark.parametrize("N,K,nb,gs,M", [
@@ -184,7 +187,8 @@ def test_config3_llama13b_block_real_bcq(gpu_device):
     _assert_close(run_block(gpu_device, bW, alpha, x, 8, orc.ALPHA_F16), want)
     # dense path from the ON-DISK tensors (dequantise, transpose, matmul)
     W = orc.dequant_lat_disk(p.disk_bWeight.cpu().numpy(), p.disk_alpha.cpu().numpy())
-    _assert_close(run_block(gpu_device, bW, alpha, x, 8, orc.ALPHA_F16), orc.dense_gemv_np(W, x.numpy()))
+    _assert_close(run_block(gpu_device, bW, alpha, x, 8, orc.ALPHA_F16), orc.dense_gemv_np(W, x.numpy()),
+                  margin=0.25)
 
 
 @pytest.mark.parametrize("N,K", workload.LLAMA2_13B_SHAPES[1:])
