@@ -45,7 +45,7 @@ def parse_args():
     ap.add_argument("--layers", type=int, default=N_LAYERS, help="distinct decoder blocks in the weight pool")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying a HIP graph")
-    ap.add_argument("--shape-table", action="store_true", help="also time every shape alone, hot and rotating")
+    ap.add_argument("--no-shape-table", action="store_true", help="skip timing every shape alone")
     ap.add_argument("--profile-shape", type=str, default="",
                     help="N,K[,nb[,iters]]: only launch this shape repeatedly (for rocprofv3 runs) and exit")
     ap.add_argument("--profile-copy", type=int, default=0,
@@ -159,75 +159,123 @@ def main():
         if rel > 2e-3 or mad > 1e-2:
             raise SystemExit(f"parity failure on {g.N}x{g.K}: rel_l2={rel} max={mad}")
 
-    # ---- the timed step -----------------------------------------------------
-    def one_step_eager():
+    # ---- launch sequences ---------------------------------------------------------
+    grouped = lib.lutgemm_gemv_rowwise_f16_grouped
+
+    def group_args(gs):
+        arr = (native.RowwiseProblem * len(gs))()
+        for i, g in enumerate(gs):
+            arr[i] = native.RowwiseProblem(g.bW.data_ptr(), g.alpha.data_ptr(), g.x.data_ptr(),
+                                           g.out.data_ptr(), g.N, g.K, g.nb, g.groups, 1)
+        return arr
+
+    def run_group(arr):
+        rc = grouped(len(arr), arr, sp)
+        if rc:
+            raise RuntimeError(lib.lutgemm_strerror(rc).decode())
+
+    blocks = [pool[i:i + 7] for i in range(0, len(pool), 7)]
+    # dependency-respecting fusion inside a decoder block: [q,k,v] [o] [gate,up] [down]
+    fused4 = [[group_args(b[0:3]), group_args(b[3:4]), group_args(b[4:6]), group_args(b[6:7])] for b in blocks]
+    # the whole 7-matrix sequence as one launch (no dependencies between the seven in this benchmark)
+    fused1 = [[group_args(b)] for b in blocks]
+
+    def seq_plain():
         for g in pool:
             run(g, sp)
 
-    with torch.cuda.stream(stream):
-        one_step_eager()                      # sizes the workspace of this stream before any capture
-    stream.synchronize()
+    def seq_fused(groups):
+        def f():
+            for blk in groups:
+                for arr in blk:
+                    run_group(arr)
+        return f
 
-    graph = None
-    if not args.no_graph:
-        graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(graph, stream=stream):
-            one_step_eager()
+    def capture(fn):
+        with torch.cuda.stream(stream):
+            fn()                              # sizes this stream's workspace before any capture
+        stream.synchronize()
+        if args.no_graph:
+            return None
+        gr = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(gr, stream=stream):
+            fn()
+        return gr
 
-    def step():
-        if graph is not None:
-            graph.replay()
-        else:
+    def timed(fn, gr, steps, warmup):
+        """(wall ms/step, device ms/step): wall clock between synchronisations and
+        HIP events recorded on the launch stream around the same region."""
+        def step():
             with torch.cuda.stream(stream):
-                one_step_eager()
+                if gr is not None:
+                    gr.replay()
+                else:
+                    fn()
+        for _ in range(warmup):
+            step()
+        torch.cuda.synchronize()
+        ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        t_start = time.perf_counter()
+        with torch.cuda.stream(stream):
+            ev0.record(stream)
+        for _ in range(steps):
+            step()
+        with torch.cuda.stream(stream):
+            ev1.record(stream)
+        torch.cuda.synchronize()
+        wall = (time.perf_counter() - t_start) * 1e3 / steps
+        return wall, ev0.elapsed_time(ev1) / steps
 
-    for _ in range(args.warmup):
-        step()
-    torch.cuda.synchronize()
-    ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    t_start = time.perf_counter()
-    with torch.cuda.stream(stream):
-        ev0.record(stream)
-    for _ in range(args.steps):
-        step()
-    with torch.cuda.stream(stream):
-        ev1.record(stream)
-    torch.cuda.synchronize()
-    wall_s = time.perf_counter() - t_start
-    dev_ms = ev0.elapsed_time(ev1)            # HIP events on the launch stream
-
-    ms_per_step = wall_s * 1e3 / args.steps
-    dev_ms_per_step = dev_ms / args.steps
+    # ---- the timed step: 224 separate launches, the drop-in call pattern -----------
+    graph = capture(seq_plain)
+    ms_per_step, dev_ms_per_step = timed(seq_plain, graph, args.steps, args.warmup)
     us_per_call = dev_ms_per_step * 1e3 / calls_per_step
     achieved_gbs = step_bytes / (dev_ms_per_step * 1e-3) / 1e9
 
-    # ---- optional per-shape table -------------------------------------------
+    # ---- the same step with fused launches --------------------------------------------
+    fused = {}
+    for label, groups, launches in (("fused_qkv_o_gateup_down", fused4, 4 * len(blocks)),
+                                    ("fused_7_in_1", fused1, len(blocks))):
+        f = seq_fused(groups)
+        gr = capture(f)
+        _, dms = timed(f, gr, args.steps, args.warmup)
+        gbs = step_bytes / (dms * 1e-3) / 1e9
+        fused[label] = {"launches_per_step": launches, "device_ms_per_step": round(dms, 5),
+                        "us_per_launch": round(dms * 1e3 / launches, 3),
+                        "us_per_gemv": round(dms * 1e3 / calls_per_step, 4),
+                        "achieved_GBps": round(gbs, 1), "frac_hbm_peak": round(gbs / HBM_PEAK_GBS, 4),
+                        "decode_tokens_per_s_linears_only": round(1e3 / dms, 1)}
+    # parity of the fused path (outputs accumulate: clear, run once, compare with a plain call)
+    for g in pool[:7]:
+        g.out.zero_()
+    with torch.cuda.stream(stream):
+        run_group(fused1[0][0])
+    stream.synchronize()
+    fused_out = [g.out.clone() for g in pool[:7]]
+    for g in pool[:7]:
+        g.out.zero_()
+    with torch.cuda.stream(stream):
+        for g in pool[:7]:
+            run(g, sp)
+    stream.synchronize()
+    parity["fused_equals_plain_bitwise"] = all(torch.equal(a, g.out) for a, g in zip(fused_out, pool[:7]))
+    if not parity["fused_equals_plain_bitwise"]:
+        raise SystemExit("fused launch disagrees with separate launches")
+
+    # ---- every shape alone: hot (one buffer, cache resident) and rotating (HBM) --------
     shape_table = None
-    if args.shape_table:
+    if not args.no_shape_table:
         shape_table = {}
         for (N, K) in ((4096, 4096), (11008, 4096), (4096, 11008)):
             same = [g for g in pool if (g.N, g.K) == (N, K)]
             row = {}
             for label, seq in (("hot", [same[0]] * 64), ("rotating", (same * 8)[:max(64, len(same))])):
-                with torch.cuda.stream(stream):
-                    for g in seq[:4]:
-                        run(g, sp)
-                stream.synchronize()
-                gr = torch.cuda.CUDAGraph()
-                with torch.cuda.graph(gr, stream=stream):
+                def f(seq=seq):
                     for g in seq:
                         run(g, sp)
-                times = []
-                for _ in range(7):
-                    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-                    with torch.cuda.stream(stream):
-                        a.record(stream)
-                    gr.replay()
-                    with torch.cuda.stream(stream):
-                        b.record(stream)
-                    torch.cuda.synchronize()
-                    times.append(a.elapsed_time(b) * 1e3 / len(seq))
-                us = statistics.median(times)
+                gr = capture(f)
+                _, dms = timed(f, gr, 7, 2)
+                us = dms * 1e3 / len(seq)
                 row[label] = {"us_per_call": round(us, 3), "GBps": round(same[0].bytes / us / 1e3, 1),
                               "frac_hbm_peak": round(same[0].bytes / us / 1e3 / HBM_PEAK_GBS, 4)}
             row["algorithmic_bytes"] = same[0].bytes
@@ -279,7 +327,7 @@ def main():
         "config": {"workload": "llama2-7b linears, 3-bit BCQ, group 128, pow2 alpha, batch 1: "
                                f"{args.layers} blocks x 7 GEMVs per step over distinct weights "
                                f"({step_bytes / 1e9:.3f} GB/step)",
-                   "launch": "eager" if graph is None else "hip-graph replay",
+                   "launch": ("eager" if graph is None else "hip-graph replay") + ", one launch per GEMV",
                    "calls_per_step": calls_per_step},
         "device_ms_per_step": round(dev_ms_per_step, 5),
         "achieved_GBps": round(achieved_gbs, 1),
@@ -291,6 +339,7 @@ def main():
                      "algorithmic_bytes_per_launch": round(mean_bytes),
                      "avg_launch_us": round(us_per_call, 4)},
         "cpu_baseline": cpu,
+        "fused_launches": fused,
         "parity": parity,
         "pool_build_s": round(t_pool, 2),
     }

@@ -63,6 +63,28 @@ int lutgemm_gemv_rowwise_f16(const uint32_t *bW, const void *alpha_f16, const vo
                              void *stream);
 
 /*
+ * Several row-wise-alpha GEMVs in ONE kernel launch.  No counterpart in the
+ * reference, which launches every linear layer separately; it exists because a
+ * launch on this hardware has a fixed cost of about 2 microseconds, more than
+ * a 7B-sized GEMV needs at HBM speed, so projections that do not depend on each
+ * other (q/k/v, gate/up) are best issued together.  Each entry has the
+ * arguments and the semantics of lutgemm_gemv_rowwise_f16; bit widths and
+ * shapes may differ between entries, outputs must not overlap.
+ * 1 <= count <= LUTGEMM_MAX_GROUP.
+ */
+#define LUTGEMM_MAX_GROUP 8
+typedef struct lutgemm_rowwise_problem {
+    const uint32_t *bW;
+    const void *alpha_f16;
+    const void *x_f16;
+    void *out_f16;
+    int N, K, nb, num_groups, M;
+} lutgemm_rowwise_problem;
+
+int lutgemm_gemv_rowwise_f16_grouped(int count, const lutgemm_rowwise_problem *problems,
+                                     void *stream);
+
+/*
  * Uniform-quantisation mode of the original LUT-GEMM.
  * Replaces lutgemm_compute -> nqmv_bias -> _nqmv_bias<32>
  * (lutgemm_cuda.cpp:88-98; lutgemm_cuda_kernel.cu:287-315;

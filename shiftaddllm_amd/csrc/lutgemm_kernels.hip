@@ -19,16 +19,23 @@
 //    (h*4+q); rows of the sign matrix are read in 512-byte contiguous runs
 //    per workgroup.  At look-up step j the lane uses byte (j+q)&3 of its
 //    word, i.e. table kw*4 + ((j+q)&3) -- distinct over (kw, q).
+//  * The loads of set i+1 are issued before the look-ups of set i, so the
+//    HBM latency of a workgroup's own stream hides behind its LDS work.
 //  * Accumulation is fp32; alphas are applied with one fma per look-up
 //    (a power-of-two alpha is then an exact exponent shift).  The 8 kw-lanes
 //    of an output are reduced with cross-lane shuffles.
-//  * K is split over workgroups (grid.y).  Partial sums go to an fp32
-//    workspace; the last workgroup to finish an N-tile (ticket counter) sums
-//    them in slice order, adds the caller's fp16 output and rounds once.
-//    Deterministic, no floating-point atomics.
+//  * K is split over workgroups.  Each workgroup adds its partial sums, as
+//    64-bit fixed point (2^-32 units), into a per-output accumulator word with
+//    ONE returning atomic; the top byte of the word counts contributions, so
+//    the contributor that sees count == ksplit-1 owns the complete sum, adds
+//    the caller's fp16 output, rounds once and clears the word.  Integer
+//    addition is associative: the result does not depend on arrival order.
+//    No fences (a device-scope release costs tens of microseconds here) and
+//    no second pass.
 #include <hip/hip_runtime.h>
 #include <hip/hip_fp16.h>
 #include <stdint.h>
+#include <stdlib.h>
 
 #include <map>
 #include <mutex>
@@ -40,13 +47,20 @@ namespace {
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
-typedef float f32x4 __attribute__((ext_vector_type(4)));
 
 constexpr int kThreads = 256;
 constexpr int kSetWords = 8;               // sign words (of 32 inputs) per table set
 constexpr int kTables = 4 * kSetWords;     // 32 tables, one per LDS bank
 constexpr int kWaveCols = 32;              // outputs a wave covers per step
 constexpr int kStepCols = 4 * kWaveCols;   // outputs a workgroup covers per step
+constexpr int kMaxKSplit = 32;             // bounded by the fixed-point accumulator layout
+constexpr int kMaxGroup = LUTGEMM_MAX_GROUP;  // problems per grouped launch
+
+// fixed-point accumulator word: [63:56] contributions, [55:0] sum of (v + kBias),
+// v = partial * 2^32 with |partial| <= 2^16
+constexpr unsigned long long kCountOne = 1ull << 56;
+constexpr unsigned long long kSumMask = kCountOne - 1;
+constexpr long long kBias = 1ll << 49;
 
 enum AlphaMode : int {
     kRowF16 = 0,      // fp16 [G][nb][N]
@@ -62,21 +76,43 @@ struct Problem {
     const __half *qbias;
     const __half *x;
     __half *out;
-    float *partial;      // [ksplit][M][N] fp32, used when ksplit > 1
-    unsigned *tickets;   // [M][n_tiles], zero between launches
+    unsigned long long *accum;  // [M][N] fixed-point words, zero between launches (ksplit > 1)
     int N, K, M;
     int kwords;          // K / 32
     int nsets;           // ceil(kwords / 8)
     int sets_per_split;
     int ksplit;
+    int n_tiles;
     int group_words;     // row-wise / uniform: words per alpha group
     int R;               // block modes: row groups
     int rows_per_group;  // block modes: N / R
+    int nb;
+    int block_begin;     // grouped launches: first flat workgroup index of this problem
+    int n_blocks;        // workgroups of this problem in the flat grid
+};
+
+// Flat workgroup index (relative to the problem) -> (tile, kslice, m).
+__device__ __forceinline__ void decode_block(const Problem &p, int local, int &tile, int &kslice, int &m)
+{
+    tile = local % p.n_tiles;
+    local /= p.n_tiles;
+    kslice = local % p.ksplit;
+    m = local / p.ksplit;
+}
+
+struct Group {
+    int count;
+    Problem p[kMaxGroup];
 };
 
 __device__ __forceinline__ float half_bits_to_float(uint32_t bits16)
 {
     return __half2float(__ushort_as_half((unsigned short)bits16));
+}
+
+__device__ __forceinline__ uint32_t float_to_half_bits(float f)
+{
+    return (uint32_t)__half_as_ushort(__float2half_rn(f));
 }
 
 // Decode one block-alpha multiplier.
@@ -100,20 +136,174 @@ __device__ __forceinline__ float load_block_alpha(const void *alpha, size_t i)
     }
 }
 
+// Everything one lane needs from global memory for one table set.
 template <int NB, int NSTEPS, int MODE>
-__global__ void __launch_bounds__(kThreads) lut_gemv_kernel(const Problem p)
-{
-    __shared__ __attribute__((aligned(16))) float lut[256 * kTables];
-    __shared__ unsigned s_is_last;
+struct SetOperands {
+    u32x4 w[NSTEPS][NB];        // sign words: 4 outputs x 32 inputs per register quad
+    u32x2 a_row[NSTEPS][NB];    // row-wise: 4 fp16 alphas (one per output)
+    float a_blk[NSTEPS][NB][4]; // block: one multiplier per look-up step
+    u32x2 a_uni[NSTEPS];        // uniform: alpha per output
+    u32x2 q_uni[NSTEPS];        // uniform: q_bias per output
+    u32x4 xraw;                 // 8 activations of the chunk this thread builds a table for
+};
 
+// Issue every global load of one table set for this lane.  Branch-free on
+// purpose: out-of-range rows and columns are clamped to valid addresses instead
+// of predicated, so the loads sit in straight-line code and the compiler can
+// keep the NEXT set's loads in flight (s_waitcnt vmcnt(n), n > 0) while the
+// current set is consumed.  Clamped data is harmless: tables of inputs beyond K
+// are all zero, and outputs beyond N are never written.
+template <int NB, int NSTEPS, int MODE>
+__device__ __forceinline__ void load_set(SetOperands<NB, NSTEPS, MODE> &r, const Problem &p,
+                                         const __half *x, int set, int kw, int q, int n_lane, int tb)
+{
+    const int row = min(set * kSetWords + kw, p.kwords - 1);
+#pragma unroll
+    for (int s = 0; s < NSTEPS; ++s) {
+        const int n = min(n_lane + s * kStepCols, p.N - 4);
+#pragma unroll
+        for (int b = 0; b < NB; ++b) {
+            const u32x4 *src = (const u32x4 *)(p.W + ((size_t)row * NB + b) * p.N + n);
+            r.w[s][b] = __builtin_nontemporal_load(src);
+        }
+        if constexpr (MODE == kRowF16) {
+            const int g = row / p.group_words;
+#pragma unroll
+            for (int b = 0; b < NB; ++b)
+                r.a_row[s][b] = *(const u32x2 *)((const __half *)p.alpha + ((size_t)g * NB + b) * p.N + n);
+        } else if constexpr (MODE == kUniformF16) {
+            const int g = row / p.group_words;
+            r.a_uni[s] = *(const u32x2 *)((const __half *)p.alpha + (size_t)g * p.N + n);
+            r.q_uni[s] = *(const u32x2 *)(p.qbias + (size_t)g * p.N + n);
+        } else {
+            const int rg = n / p.rows_per_group;
+#pragma unroll
+            for (int b = 0; b < NB; ++b)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const int chunk = row * 4 + ((j + q) & 3);
+                    r.a_blk[s][b][j] = load_block_alpha<MODE>(p.alpha, ((size_t)chunk * NB + b) * p.R + rg);
+                }
+        }
+    }
+    const int k0 = (set * kTables + tb) * 8;
+    const u32x4 xr = *(const u32x4 *)(x + min(k0, p.K - 8));
+    const bool live = k0 < p.K;
+    r.xraw.x = live ? xr.x : 0u;
+    r.xraw.y = live ? xr.y : 0u;
+    r.xraw.z = live ? xr.z : 0u;
+    r.xraw.w = live ? xr.w : 0u;
+}
+
+// Build the 32 tables of one set, then run this lane's look-ups against them.
+template <int NB, int NSTEPS, int MODE>
+__device__ __forceinline__ void consume_set(const SetOperands<NB, NSTEPS, MODE> &cur, float *lut,
+                                            float (&acc)[NSTEPS][4], const int (&bank)[4], int q,
+                                            int tb, int eb)
+{
+    // ---- build: this thread writes entries eb*32 .. +31 of table tb -----------
+    float x2[8];  // 2 * x
+    float base = 0.0f;
+    {
+        const uint32_t r4[4] = {cur.xraw.x, cur.xraw.y, cur.xraw.z, cur.xraw.w};
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const float lo = half_bits_to_float(r4[j] & 0xffffu);
+            const float hi = half_bits_to_float(r4[j] >> 16);
+            x2[2 * j] = lo + lo;
+            x2[2 * j + 1] = hi + hi;
+            base -= lo + hi;  // entry 0 = -sum x
+        }
+    }
+    __syncthreads();  // look-ups of the previous set are done with the tables
+    {
+        float top = base;  // bits 5..7 of the entry index come from eb
+#pragma unroll
+        for (int j = 5; j < 8; ++j)
+            if ((eb >> (j - 5)) & 1) top += x2[j];
+        float *col = lut + (eb * 32) * kTables + tb;
+#pragma unroll
+        for (int sb = 0; sb < 4; ++sb) {  // bits 3,4 fixed per sub-block: 4 short chains
+            float v = top;
+            if (sb & 1) v += x2[3];
+            if (sb & 2) v += x2[4];
+            unsigned gray = 0;
+            col[(sb * 8) * kTables] = v;
+#pragma unroll
+            for (int i = 1; i < 8; ++i) {
+                const int bit = __builtin_ctz(i);
+                gray ^= 1u << bit;
+                v += ((gray >> bit) & 1u) ? x2[bit] : -x2[bit];
+                col[(sb * 8 + gray) * kTables] = v;
+            }
+        }
+    }
+    __syncthreads();
+
+    // ---- look-ups, software pipelined in units of 16 (one bit plane of one step):
+    // the LDS reads of unit u+1 are issued before the fmas of unit u
+    constexpr int kUnits = NSTEPS * NB;
+    float val[2][16];
+    auto issue = [&](int u, float (&v)[16]) {
+        const int s = u / NB, b = u % NB;
+        const uint32_t w4[4] = {cur.w[s][b].x, cur.w[s][b].y, cur.w[s][b].z, cur.w[s][b].w};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const uint32_t w = __builtin_rotateright32(w4[i], 8 * q);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) v[4 * i + j] = lut[((w >> (8 * j)) & 255u) * kTables + bank[j]];
+        }
+    };
+    auto retire = [&](int u, const float (&v)[16]) {
+        const int s = u / NB, b = u % NB;
+        [[maybe_unused]] const uint32_t ar[2] = {cur.a_row[s][b].x, cur.a_row[s][b].y};
+        [[maybe_unused]] const uint32_t au[2] = {cur.a_uni[s].x, cur.a_uni[s].y};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            float a = 0.0f;
+            if constexpr (MODE == kRowF16)
+                a = half_bits_to_float((ar[i >> 1] >> (16 * (i & 1))) & 0xffffu);
+            else if constexpr (MODE == kUniformF16)
+                a = half_bits_to_float((au[i >> 1] >> (16 * (i & 1))) & 0xffffu) * (1.0f / (float)(2 << b));
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                if constexpr (MODE == kBlockF16 || MODE == kBlockShiftU16 || MODE == kBlockApotI8)
+                    a = cur.a_blk[s][b][j];
+                acc[s][i] = fmaf(v[4 * i + j], a, acc[s][i]);
+            }
+        }
+    };
+    issue(0, val[0]);
+    if constexpr (MODE == kUniformF16) {
+        float sum_x = 0.0f;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) sum_x += lut[255 * kTables + bank[j]];
+#pragma unroll
+        for (int s = 0; s < NSTEPS; ++s) {
+            const uint32_t rq[2] = {cur.q_uni[s].x, cur.q_uni[s].y};
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                acc[s][i] = fmaf(half_bits_to_float((rq[i >> 1] >> (16 * (i & 1))) & 0xffffu), sum_x, acc[s][i]);
+        }
+    }
+#pragma unroll
+    for (int u = 0; u < kUnits; ++u) {
+        if (u + 1 < kUnits) issue(u + 1, val[(u + 1) & 1]);
+        retire(u, val[u & 1]);
+    }
+}
+
+// One workgroup's share: N-tile `tile`, K-slice `kslice`, activation row `m`.
+template <int NB, int NSTEPS, int MODE>
+__device__ __forceinline__ void gemv_tile(const Problem &p, int tile, int kslice, int m, float *lut)
+{
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = tid >> 6;
     const int q = lane & 3;
     const int kw = (lane >> 2) & 7;
     const int h = lane >> 5;
-    const int m = blockIdx.z;
-    const int tile0 = blockIdx.x * (kStepCols * NSTEPS);
+    const int tile0 = tile * (kStepCols * NSTEPS);
     const int n_lane = tile0 + wave * kWaveCols + (h * 4 + q) * 4;  // + s*kStepCols
 
     const __half *x = p.x + (size_t)m * p.K;
@@ -133,172 +323,40 @@ __global__ void __launch_bounds__(kThreads) lut_gemv_kernel(const Problem p)
     const int tb = tid & 31;  // table (bank)
     const int eb = tid >> 5;  // entries eb*32 .. eb*32+31
 
-    const int set_begin = blockIdx.y * p.sets_per_split;
+    const int set_begin = kslice * p.sets_per_split;
     const int set_end = min(set_begin + p.sets_per_split, p.nsets);
 
-    for (int set = set_begin; set < set_end; ++set) {
-        // ---- 1. issue the streaming loads for this set -------------------------
-        const int row = set * kSetWords + kw;
-        const bool row_ok = row < p.kwords;
-        u32x4 wreg[NSTEPS][NB];
-#pragma unroll
-        for (int s = 0; s < NSTEPS; ++s) {
-            const int n = n_lane + s * kStepCols;
-            const bool ok = row_ok && n < p.N;
-#pragma unroll
-            for (int b = 0; b < NB; ++b) {
-                if (ok) {
-                    const u32x4 *src = (const u32x4 *)(p.W + ((size_t)row * NB + b) * p.N + n);
-                    wreg[s][b] = __builtin_nontemporal_load(src);
-                } else {
-                    wreg[s][b] = (u32x4){0u, 0u, 0u, 0u};
-                }
-            }
-        }
+    // two operand buffers used alternately, so that no register copy (which would
+    // have to wait for the loads) sits between a set's loads and its use
+    SetOperands<NB, NSTEPS, MODE> opA, opB;
+    load_set<NB, NSTEPS, MODE>(opA, p, x, set_begin, kw, q, n_lane, tb);
 
-        // alpha operands
-        [[maybe_unused]] float a_row[NSTEPS][NB][4];    // row-wise: per (bit, output)
-        [[maybe_unused]] float a_blk[NSTEPS][NB][4];    // block: per (bit, look-up step)
-        [[maybe_unused]] float a_uni[NSTEPS][4];        // uniform: alpha per output
-        [[maybe_unused]] float q_uni[NSTEPS][4];        // uniform: q_bias per output
-        if constexpr (MODE == kRowF16) {
-            const int g = row / p.group_words;
+    // the caller's output, needed only by whoever completes a sum: fetched now,
+    // off the critical path
+    u32x2 out_raw[NSTEPS];
+    __half *out = p.out + (size_t)m * p.N;
 #pragma unroll
-            for (int s = 0; s < NSTEPS; ++s) {
-                const int n = n_lane + s * kStepCols;
-                const bool ok = row_ok && n < p.N;
-#pragma unroll
-                for (int b = 0; b < NB; ++b) {
-                    u32x2 raw = (u32x2){0u, 0u};
-                    if (ok)
-                        raw = *(const u32x2 *)((const __half *)p.alpha + ((size_t)g * NB + b) * p.N + n);
-                    a_row[s][b][0] = half_bits_to_float(raw.x & 0xffffu);
-                    a_row[s][b][1] = half_bits_to_float(raw.x >> 16);
-                    a_row[s][b][2] = half_bits_to_float(raw.y & 0xffffu);
-                    a_row[s][b][3] = half_bits_to_float(raw.y >> 16);
-                }
-            }
-        } else if constexpr (MODE == kUniformF16) {
-            const int g = row / p.group_words;
-#pragma unroll
-            for (int s = 0; s < NSTEPS; ++s) {
-                const int n = n_lane + s * kStepCols;
-                const bool ok = row_ok && n < p.N;
-                u32x2 ra = (u32x2){0u, 0u}, rq = (u32x2){0u, 0u};
-                if (ok) {
-                    ra = *(const u32x2 *)((const __half *)p.alpha + (size_t)g * p.N + n);
-                    rq = *(const u32x2 *)(p.qbias + (size_t)g * p.N + n);
-                }
-                a_uni[s][0] = half_bits_to_float(ra.x & 0xffffu);
-                a_uni[s][1] = half_bits_to_float(ra.x >> 16);
-                a_uni[s][2] = half_bits_to_float(ra.y & 0xffffu);
-                a_uni[s][3] = half_bits_to_float(ra.y >> 16);
-                q_uni[s][0] = half_bits_to_float(rq.x & 0xffffu);
-                q_uni[s][1] = half_bits_to_float(rq.x >> 16);
-                q_uni[s][2] = half_bits_to_float(rq.y & 0xffffu);
-                q_uni[s][3] = half_bits_to_float(rq.y >> 16);
-            }
-        } else {
-#pragma unroll
-            for (int s = 0; s < NSTEPS; ++s) {
-                const int n = n_lane + s * kStepCols;
-                const bool ok = row_ok && n < p.N;
-                const int r = ok ? n / p.rows_per_group : 0;
-#pragma unroll
-                for (int b = 0; b < NB; ++b)
-#pragma unroll
-                    for (int j = 0; j < 4; ++j) {
-                        const int chunk = row * 4 + ((j + q) & 3);
-                        a_blk[s][b][j] =
-                            ok ? load_block_alpha<MODE>(p.alpha, ((size_t)chunk * NB + b) * p.R + r)
-                               : 0.0f;
-                    }
-            }
-        }
+    for (int s = 0; s < NSTEPS; ++s)
+        out_raw[s] = *(const u32x2 *)(out + min(n_lane + s * kStepCols, p.N - 4));
 
-        // activations of the chunk whose table this thread helps to build
-        float x2[8];  // 2 * x
-        float base = 0.0f;
-        {
-            const int k0 = (set * kTables + tb) * 8;
-            u32x4 raw = (u32x4){0u, 0u, 0u, 0u};
-            if (k0 < p.K) raw = *(const u32x4 *)(x + k0);
-            const uint32_t r4[4] = {raw.x, raw.y, raw.z, raw.w};
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const float lo = half_bits_to_float(r4[j] & 0xffffu);
-                const float hi = half_bits_to_float(r4[j] >> 16);
-                x2[2 * j] = lo + lo;
-                x2[2 * j + 1] = hi + hi;
-                base -= lo + hi;  // entry 0 = -sum x
-            }
+    for (int set = set_begin;;) {
+        if (set + 1 >= set_end) {
+            consume_set<NB, NSTEPS, MODE>(opA, lut, acc, bank, q, tb, eb);
+            break;
         }
-
-        __syncthreads();  // look-ups of the previous set are done with the tables
-
-        // ---- 2. build: this thread writes entries eb*32 .. +31 of table tb ----
-        {
-            // bits 5..7 of the entry index come from eb
-            float top = base;
-#pragma unroll
-            for (int j = 5; j < 8; ++j)
-                if ((eb >> (j - 5)) & 1) top += x2[j];
-            float *col = lut + (eb * 32) * kTables + tb;
-#pragma unroll
-            for (int sb = 0; sb < 4; ++sb) {  // bits 3,4 fixed per sub-block: 4 short chains
-                float v = top;
-                if (sb & 1) v += x2[3];
-                if (sb & 2) v += x2[4];
-                unsigned gray = 0;
-                col[(sb * 8) * kTables] = v;
-#pragma unroll
-                for (int i = 1; i < 8; ++i) {
-                    const int bit = __builtin_ctz(i);
-                    gray ^= 1u << bit;
-                    v += ((gray >> bit) & 1u) ? x2[bit] : -x2[bit];
-                    col[(sb * 8 + gray) * kTables] = v;
-                }
-            }
+        load_set<NB, NSTEPS, MODE>(opB, p, x, set + 1, kw, q, n_lane, tb);
+        consume_set<NB, NSTEPS, MODE>(opA, lut, acc, bank, q, tb, eb);
+        ++set;
+        if (set + 1 >= set_end) {
+            consume_set<NB, NSTEPS, MODE>(opB, lut, acc, bank, q, tb, eb);
+            break;
         }
-        __syncthreads();
-
-        // ---- 3. look-ups ---------------------------------------------------
-        [[maybe_unused]] float sum_x = 0.0f;
-        if constexpr (MODE == kUniformF16) {
-#pragma unroll
-            for (int j = 0; j < 4; ++j) sum_x += lut[255 * kTables + bank[j]];
-        }
-#pragma unroll
-        for (int s = 0; s < NSTEPS; ++s) {
-            if constexpr (MODE == kUniformF16) {
-#pragma unroll
-                for (int i = 0; i < 4; ++i) acc[s][i] = fmaf(q_uni[s][i], sum_x, acc[s][i]);
-            }
-#pragma unroll
-            for (int b = 0; b < NB; ++b) {
-                const uint32_t w4[4] = {wreg[s][b].x, wreg[s][b].y, wreg[s][b].z, wreg[s][b].w};
-#pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    const uint32_t w = __builtin_rotateright32(w4[i], 8 * q);
-#pragma unroll
-                    for (int j = 0; j < 4; ++j) {
-                        const uint32_t idx = (w >> (8 * j)) & 255u;
-                        const float v = lut[idx * kTables + bank[j]];
-                        float a;
-                        if constexpr (MODE == kRowF16)
-                            a = a_row[s][b][i];
-                        else if constexpr (MODE == kUniformF16)
-                            a = a_uni[s][i] * (1.0f / (float)(2 << b));
-                        else
-                            a = a_blk[s][b][j];
-                        acc[s][i] = fmaf(v, a, acc[s][i]);
-                    }
-                }
-            }
-        }
+        load_set<NB, NSTEPS, MODE>(opA, p, x, set + 1, kw, q, n_lane, tb);
+        consume_set<NB, NSTEPS, MODE>(opB, lut, acc, bank, q, tb, eb);
+        ++set;
     }
 
-    // ---- 4. reduce the 8 kw-lanes of each output, write ---------------------
+    // ---- reduce the 8 kw-lanes of each output --------------------------------
 #pragma unroll
     for (int s = 0; s < NSTEPS; ++s)
 #pragma unroll
@@ -309,69 +367,94 @@ __global__ void __launch_bounds__(kThreads) lut_gemv_kernel(const Problem p)
             v += __shfl_xor(v, 16);
             acc[s][i] = v;
         }
+    if (kw != 0) return;
 
-    __half *out = p.out + (size_t)m * p.N;
     if (p.ksplit == 1) {
-        if (kw == 0) {
 #pragma unroll
-            for (int s = 0; s < NSTEPS; ++s) {
-                const int n = n_lane + s * kStepCols;
-                if (n < p.N) {
-                    u32x2 raw = *(const u32x2 *)(out + n);
-                    const float o0 = half_bits_to_float(raw.x & 0xffffu) + acc[s][0];
-                    const float o1 = half_bits_to_float(raw.x >> 16) + acc[s][1];
-                    const float o2 = half_bits_to_float(raw.y & 0xffffu) + acc[s][2];
-                    const float o3 = half_bits_to_float(raw.y >> 16) + acc[s][3];
-                    raw.x = (uint32_t)__half_as_ushort(__float2half_rn(o0)) |
-                            ((uint32_t)__half_as_ushort(__float2half_rn(o1)) << 16);
-                    raw.y = (uint32_t)__half_as_ushort(__float2half_rn(o2)) |
-                            ((uint32_t)__half_as_ushort(__float2half_rn(o3)) << 16);
-                    *(u32x2 *)(out + n) = raw;
-                }
+        for (int s = 0; s < NSTEPS; ++s) {
+            const int n = n_lane + s * kStepCols;
+            if (n < p.N) {
+                u32x2 raw = out_raw[s];
+                const float o0 = half_bits_to_float(raw.x & 0xffffu) + acc[s][0];
+                const float o1 = half_bits_to_float(raw.x >> 16) + acc[s][1];
+                const float o2 = half_bits_to_float(raw.y & 0xffffu) + acc[s][2];
+                const float o3 = half_bits_to_float(raw.y >> 16) + acc[s][3];
+                raw.x = float_to_half_bits(o0) | (float_to_half_bits(o1) << 16);
+                raw.y = float_to_half_bits(o2) | (float_to_half_bits(o3) << 16);
+                *(u32x2 *)(out + n) = raw;
             }
         }
         return;
     }
 
-    float *partial = p.partial + ((size_t)blockIdx.y * p.M + m) * p.N;
-    if (kw == 0) {
+    // ---- K-split: one returning fixed-point atomic per output -------------------
+    unsigned long long *accum = p.accum + (size_t)m * p.N;
+    unsigned long long contrib[NSTEPS][4], old[NSTEPS][4];
 #pragma unroll
-        for (int s = 0; s < NSTEPS; ++s) {
-            const int n = n_lane + s * kStepCols;
+    for (int s = 0; s < NSTEPS; ++s) {
+        const int n = n_lane + s * kStepCols;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            // non-finite or out-of-range partial sums saturate (fp16 rounds them to inf)
+            float v = acc[s][i];
+            v = (v == v) ? v : 65536.0f;
+            v = fminf(fmaxf(v, -65536.0f), 65536.0f);
+            const long long fx = __double2ll_rn((double)v * 4294967296.0);
+            contrib[s][i] = (unsigned long long)(fx + kBias) + kCountOne;
+            old[s][i] = 0;
             if (n < p.N)
-                *(f32x4 *)(partial + n) = (f32x4){acc[s][0], acc[s][1], acc[s][2], acc[s][3]};
+                old[s][i] = __hip_atomic_fetch_add(accum + n + i, contrib[s][i], __ATOMIC_RELAXED,
+                                                   __HIP_MEMORY_SCOPE_AGENT);
         }
     }
-    __threadfence();  // release: partials visible device-wide before the ticket
-    __syncthreads();
-    unsigned *ticket = p.tickets + (size_t)m * gridDim.x + blockIdx.x;
-    if (tid == 0) {
-        const unsigned t = atomicAdd(ticket, 1u);
-        s_is_last = (t == (unsigned)(p.ksplit - 1)) ? 1u : 0u;
-    }
-    __syncthreads();
-    if (!s_is_last) return;
-    __threadfence();  // acquire: see every other workgroup's partials
-
-    for (int quad = tid; quad < (kStepCols * NSTEPS) / 4; quad += kThreads) {
-        const int n = tile0 + quad * 4;
+#pragma unroll
+    for (int s = 0; s < NSTEPS; ++s) {
+        const int n = n_lane + s * kStepCols;
         if (n >= p.N) continue;
-        f32x4 sum = (f32x4){0.0f, 0.0f, 0.0f, 0.0f};
-        const float *src = p.partial + (size_t)m * p.N + n;
-        for (int ks = 0; ks < p.ksplit; ++ks)
-            sum += *(const f32x4 *)(src + (size_t)ks * p.M * p.N);
-        u32x2 raw = *(const u32x2 *)(out + n);
-        const float o0 = half_bits_to_float(raw.x & 0xffffu) + sum.x;
-        const float o1 = half_bits_to_float(raw.x >> 16) + sum.y;
-        const float o2 = half_bits_to_float(raw.y & 0xffffu) + sum.z;
-        const float o3 = half_bits_to_float(raw.y >> 16) + sum.w;
-        raw.x = (uint32_t)__half_as_ushort(__float2half_rn(o0)) |
-                ((uint32_t)__half_as_ushort(__float2half_rn(o1)) << 16);
-        raw.y = (uint32_t)__half_as_ushort(__float2half_rn(o2)) |
-                ((uint32_t)__half_as_ushort(__float2half_rn(o3)) << 16);
-        *(u32x2 *)(out + n) = raw;
+        const uint32_t raw2[2] = {out_raw[s].x, out_raw[s].y};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            if ((int)(old[s][i] >> 56) != p.ksplit - 1) continue;
+            // this contribution completed the sum
+            const long long total =
+                (long long)((old[s][i] + contrib[s][i]) & kSumMask) - (long long)p.ksplit * kBias;
+            const float y = (float)((double)total * (1.0 / 4294967296.0));
+            const float o = half_bits_to_float((raw2[i >> 1] >> (16 * (i & 1))) & 0xffffu) + y;
+            out[n + i] = __float2half_rn(o);
+            __hip_atomic_store(accum + n + i, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
     }
-    if (tid == 0) *ticket = 0u;  // ready for the next launch
+}
+
+template <int NB, int NSTEPS, int MODE>
+__global__ void __launch_bounds__(kThreads) lut_gemv_kernel(const Problem p)
+{
+    __shared__ __attribute__((aligned(16))) float lut[256 * kTables];
+    int tile, kslice, m;
+    decode_block(p, (int)blockIdx.x, tile, kslice, m);
+    gemv_tile<NB, NSTEPS, MODE>(p, tile, kslice, m, lut);
+}
+
+// Several row-wise problems in one launch (flat 1-D grid).  Bit widths may
+// differ between the problems of a group.
+template <int NSTEPS>
+__global__ void __launch_bounds__(kThreads) lut_gemv_group_kernel(const Group g)
+{
+    __shared__ __attribute__((aligned(16))) float lut[256 * kTables];
+    const int b = blockIdx.x;
+    int pi = 0;
+#pragma unroll
+    for (int i = 1; i < kMaxGroup; ++i)
+        if (i < g.count && b >= g.p[i].block_begin) pi = i;
+    const Problem &p = g.p[pi];
+    int tile, kslice, m;
+    decode_block(p, b - p.block_begin, tile, kslice, m);
+    switch (p.nb) {
+    case 1: gemv_tile<1, NSTEPS, kRowF16>(p, tile, kslice, m, lut); break;
+    case 2: gemv_tile<2, NSTEPS, kRowF16>(p, tile, kslice, m, lut); break;
+    case 3: gemv_tile<3, NSTEPS, kRowF16>(p, tile, kslice, m, lut); break;
+    default: gemv_tile<4, NSTEPS, kRowF16>(p, tile, kslice, m, lut); break;
+    }
 }
 
 __global__ void __launch_bounds__(256) copy_kernel(u32x4 *dst, const u32x4 *src, size_t n16)
@@ -388,10 +471,8 @@ __global__ void __launch_bounds__(256) copy_kernel(u32x4 *dst, const u32x4 *src,
 thread_local int g_last_hip_error = 0;
 
 struct Workspace {
-    float *partial = nullptr;
-    size_t partial_floats = 0;
-    unsigned *tickets = nullptr;
-    size_t n_tickets = 0;
+    unsigned long long *accum = nullptr;
+    size_t words = 0;
 };
 
 std::mutex g_ws_mutex;
@@ -403,81 +484,89 @@ int hip_fail(hipError_t e)
     return LUTGEMM_EHIP;
 }
 
-// Grow-only workspace per (device, stream).  Launches on one stream are
-// ordered, so a stream can share one workspace across calls.
-int get_workspace(hipStream_t stream, size_t partial_floats, size_t n_tickets, Workspace *out)
+// Grow-only, zero-initialised accumulator words per (device, stream).  Launches
+// on one stream are ordered and every launch leaves its words at zero again, so
+// a stream shares one workspace across calls.  Growing synchronises the stream
+// and allocates: do a first call of each shape before capturing a graph.
+int get_workspace(hipStream_t stream, size_t words, unsigned long long **out)
 {
     int dev = 0;
     hipError_t e = hipGetDevice(&dev);
     if (e != hipSuccess) return hip_fail(e);
     std::lock_guard<std::mutex> lock(g_ws_mutex);
     Workspace &ws = g_workspaces[std::make_pair(dev, stream)];
-    if (ws.partial_floats < partial_floats || ws.n_tickets < n_tickets) {
-        // work queued on the stream may still use the old buffers
+    if (ws.words < words) {
+        e = hipStreamSynchronize(stream);  // queued work may still use the old buffer
+        if (e != hipSuccess) return hip_fail(e);
+        if (ws.accum) (void)hipFree(ws.accum);
+        ws.accum = nullptr;
+        ws.words = 0;
+        size_t want = words < (1u << 18) ? (1u << 18) : words;
+        e = hipMalloc((void **)&ws.accum, want * sizeof(unsigned long long));
+        if (e != hipSuccess) {
+            g_last_hip_error = (int)e;
+            return LUTGEMM_ENOMEM;
+        }
+        e = hipMemsetAsync(ws.accum, 0, want * sizeof(unsigned long long), stream);
+        if (e != hipSuccess) return hip_fail(e);
         e = hipStreamSynchronize(stream);
         if (e != hipSuccess) return hip_fail(e);
-        if (ws.partial_floats < partial_floats) {
-            if (ws.partial) (void)hipFree(ws.partial);
-            ws.partial = nullptr;
-            ws.partial_floats = 0;
-            size_t want = partial_floats < (1u << 20) ? (1u << 20) : partial_floats;
-            e = hipMalloc((void **)&ws.partial, want * sizeof(float));
-            if (e != hipSuccess) { g_last_hip_error = (int)e; return LUTGEMM_ENOMEM; }
-            ws.partial_floats = want;
-        }
-        if (ws.n_tickets < n_tickets) {
-            if (ws.tickets) (void)hipFree(ws.tickets);
-            ws.tickets = nullptr;
-            ws.n_tickets = 0;
-            size_t want = n_tickets < 4096 ? 4096 : n_tickets;
-            e = hipMalloc((void **)&ws.tickets, want * sizeof(unsigned));
-            if (e != hipSuccess) { g_last_hip_error = (int)e; return LUTGEMM_ENOMEM; }
-            e = hipMemsetAsync(ws.tickets, 0, want * sizeof(unsigned), stream);
-            if (e != hipSuccess) return hip_fail(e);
-            e = hipStreamSynchronize(stream);
-            if (e != hipSuccess) return hip_fail(e);
-            ws.n_tickets = want;
-        }
+        ws.words = want;
     }
-    *out = ws;
+    *out = ws.accum;
     return LUTGEMM_OK;
 }
 
-struct Plan {
-    int nsteps;   // 1, 2 or 4
-    int ksplit;
-    int sets_per_split;
-    int n_tiles;
-};
-
-// Pick the N-tile and the K-split so that the launch has a few workgroups per
-// CU (256 CUs) while each workgroup still does enough look-ups per table built.
-Plan make_plan(int N, int K, int M)
+int env_int(const char *name, int fallback)
 {
-    const int nsets = (K / 32 + kSetWords - 1) / kSetWords;
-    const long target_blocks = 1024;
-    Plan best{};
-    int nsteps = 2;
-    if (N <= 128) nsteps = 1;
-    const int n_tiles = (N + kStepCols * nsteps - 1) / (kStepCols * nsteps);
-    long want = target_blocks / ((long)n_tiles * M);
+    const char *v = getenv(name);
+    return (v && *v) ? atoi(v) : fallback;
+}
+
+// Tuning knobs (read once): LUTGEMM_TARGET_BLOCKS = workgroups a launch aims
+// for, LUTGEMM_NSTEPS = 1 or 2 output steps per workgroup.
+int target_blocks()
+{
+    static const int v = env_int("LUTGEMM_TARGET_BLOCKS", 1024);
+    return v;
+}
+int forced_nsteps()
+{
+    static const int v = env_int("LUTGEMM_NSTEPS", 0);
+    return v;
+}
+
+// Pick the N-tile and the K-split so that `want_blocks` workgroups exist while
+// each still does enough look-ups per table built.
+void plan_problem(Problem &p, int nsteps, long want_blocks)
+{
+    p.n_tiles = (p.N + kStepCols * nsteps - 1) / (kStepCols * nsteps);
+    long want = want_blocks / ((long)p.n_tiles * p.M);
     if (want < 1) want = 1;
-    if (want > nsets) want = nsets;
-    int sets_per_split = (nsets + (int)want - 1) / (int)want;
-    int ksplit = (nsets + sets_per_split - 1) / sets_per_split;
-    best.nsteps = nsteps;
-    best.ksplit = ksplit;
-    best.sets_per_split = sets_per_split;
-    best.n_tiles = n_tiles;
-    return best;
+    if (want > p.nsets) want = p.nsets;
+    if (want > kMaxKSplit) want = kMaxKSplit;
+    p.sets_per_split = (p.nsets + (int)want - 1) / (int)want;
+    p.ksplit = (p.nsets + p.sets_per_split - 1) / p.sets_per_split;
+    p.n_blocks = p.n_tiles * p.ksplit * p.M;
+}
+
+int pick_nsteps(int N)
+{
+    // One step (128 outputs per workgroup) measured faster than two on every
+    // shape tried: twice the workgroups to spread the stream over, and a shorter
+    // tail, outweigh building each table for half as many look-ups.
+    const int f = forced_nsteps();
+    if (f == 1 || f == 2) return f;
+    (void)N;
+    return 1;
 }
 
 template <int NB, int MODE>
-int launch_nb(const Problem &p, const Plan &plan, hipStream_t stream)
+int launch_nb(const Problem &p, int nsteps, hipStream_t stream)
 {
-    dim3 grid((unsigned)plan.n_tiles, (unsigned)plan.ksplit, (unsigned)p.M);
+    dim3 grid((unsigned)p.n_blocks);
     dim3 block(kThreads);
-    if (plan.nsteps == 1)
+    if (nsteps == 1)
         hipLaunchKernelGGL((lut_gemv_kernel<NB, 1, MODE>), grid, block, 0, stream, p);
     else
         hipLaunchKernelGGL((lut_gemv_kernel<NB, 2, MODE>), grid, block, 0, stream, p);
@@ -487,21 +576,22 @@ int launch_nb(const Problem &p, const Plan &plan, hipStream_t stream)
 }
 
 template <int MODE>
-int launch_mode(const Problem &p, int nb, const Plan &plan, hipStream_t stream)
+int launch_mode(const Problem &p, int nsteps, hipStream_t stream)
 {
-    switch (nb) {
-    case 1: return launch_nb<1, MODE>(p, plan, stream);
-    case 2: return launch_nb<2, MODE>(p, plan, stream);
-    case 3: return launch_nb<3, MODE>(p, plan, stream);
-    case 4: return launch_nb<4, MODE>(p, plan, stream);
+    switch (p.nb) {
+    case 1: return launch_nb<1, MODE>(p, nsteps, stream);
+    case 2: return launch_nb<2, MODE>(p, nsteps, stream);
+    case 3: return launch_nb<3, MODE>(p, nsteps, stream);
+    case 4: return launch_nb<4, MODE>(p, nsteps, stream);
     default: return LUTGEMM_EINVAL;
     }
 }
 
 bool aligned(const void *ptr, size_t a) { return ((uintptr_t)ptr & (a - 1)) == 0; }
 
-int run(int mode, const uint32_t *bW, const void *alpha, const void *qbias, const void *x,
-        void *out, int N, int K, int nb, int num_groups, int M, void *stream_v)
+// Validate one problem and fill everything but the launch plan.
+int fill_problem(Problem &p, int mode, const uint32_t *bW, const void *alpha, const void *qbias,
+                 const void *x, void *out, int N, int K, int nb, int num_groups, int M)
 {
     if (!bW || !alpha || !x || !out) return LUTGEMM_EINVAL;
     if (mode == kUniformF16 && !qbias) return LUTGEMM_EINVAL;
@@ -511,7 +601,7 @@ int run(int mode, const uint32_t *bW, const void *alpha, const void *qbias, cons
     if (M > 65535) return LUTGEMM_EINVAL;
     if (!aligned(bW, 16) || !aligned(x, 16) || !aligned(out, 8)) return LUTGEMM_EALIGN;
 
-    Problem p{};
+    p = Problem{};
     p.W = bW;
     p.alpha = alpha;
     p.qbias = (const __half *)qbias;
@@ -520,6 +610,7 @@ int run(int mode, const uint32_t *bW, const void *alpha, const void *qbias, cons
     p.N = N;
     p.K = K;
     p.M = M;
+    p.nb = nb;
     p.kwords = K / 32;
     p.nsets = (p.kwords + kSetWords - 1) / kSetWords;
     if (mode == kRowF16 || mode == kUniformF16) {
@@ -535,26 +626,28 @@ int run(int mode, const uint32_t *bW, const void *alpha, const void *qbias, cons
         p.rows_per_group = N / num_groups;
         if (p.rows_per_group % 4 != 0) return LUTGEMM_EINVAL;
     }
-    // x rows must stay 16-byte aligned for the table build
-    if (M > 1 && (K % 8) != 0) return LUTGEMM_EINVAL;
+    return LUTGEMM_OK;
+}
 
+int run(int mode, const uint32_t *bW, const void *alpha, const void *qbias, const void *x,
+        void *out, int N, int K, int nb, int num_groups, int M, void *stream_v)
+{
+    Problem p;
+    int rc = fill_problem(p, mode, bW, alpha, qbias, x, out, N, K, nb, num_groups, M);
+    if (rc != LUTGEMM_OK) return rc;
     hipStream_t stream = (hipStream_t)stream_v;
-    Plan plan = make_plan(N, K, M);
-    p.ksplit = plan.ksplit;
-    p.sets_per_split = plan.sets_per_split;
-    if (plan.ksplit > 1) {
-        Workspace ws;
-        int rc = get_workspace(stream, (size_t)plan.ksplit * M * N, (size_t)plan.n_tiles * M, &ws);
+    const int nsteps = pick_nsteps(N);
+    plan_problem(p, nsteps, target_blocks());
+    if (p.ksplit > 1) {
+        rc = get_workspace(stream, (size_t)M * N, &p.accum);
         if (rc != LUTGEMM_OK) return rc;
-        p.partial = ws.partial;
-        p.tickets = ws.tickets;
     }
     switch (mode) {
-    case kRowF16: return launch_mode<kRowF16>(p, nb, plan, stream);
-    case kBlockF16: return launch_mode<kBlockF16>(p, nb, plan, stream);
-    case kBlockShiftU16: return launch_mode<kBlockShiftU16>(p, nb, plan, stream);
-    case kBlockApotI8: return launch_mode<kBlockApotI8>(p, nb, plan, stream);
-    case kUniformF16: return launch_mode<kUniformF16>(p, nb, plan, stream);
+    case kRowF16: return launch_mode<kRowF16>(p, nsteps, stream);
+    case kBlockF16: return launch_mode<kBlockF16>(p, nsteps, stream);
+    case kBlockShiftU16: return launch_mode<kBlockShiftU16>(p, nsteps, stream);
+    case kBlockApotI8: return launch_mode<kBlockApotI8>(p, nsteps, stream);
+    case kUniformF16: return launch_mode<kUniformF16>(p, nsteps, stream);
     default: return LUTGEMM_EINVAL;
     }
 }
@@ -585,6 +678,53 @@ int lutgemm_gemv_rowwise_f16(const uint32_t *bW, const void *alpha_f16, const vo
                              void *stream)
 {
     return run(kRowF16, bW, alpha_f16, nullptr, x_f16, out_f16, N, K, nb, num_groups, M, stream);
+}
+
+int lutgemm_gemv_rowwise_f16_grouped(int count, const lutgemm_rowwise_problem *problems,
+                                     void *stream_v)
+{
+    if (!problems || count < 1 || count > kMaxGroup) return LUTGEMM_EINVAL;
+    Group g{};
+    g.count = count;
+    hipStream_t stream = (hipStream_t)stream_v;
+    size_t words = 0;
+    long total_bytes = 0;
+    for (int i = 0; i < count; ++i) {
+        const lutgemm_rowwise_problem &q = problems[i];
+        int rc = fill_problem(g.p[i], kRowF16, q.bW, q.alpha_f16, nullptr, q.x_f16, q.out_f16, q.N,
+                              q.K, q.nb, q.num_groups, q.M);
+        if (rc != LUTGEMM_OK) return rc;
+        words += (size_t)q.M * q.N;
+        total_bytes += (long)q.N * (q.K / 8) * q.nb * q.M;
+    }
+    // share the launch's workgroup budget in proportion to each problem's sign bytes
+    const long budget = (long)target_blocks() * (count > 1 ? 2 : 1);
+    int begin = 0;
+    bool any_split = false;
+    for (int i = 0; i < count; ++i) {
+        Problem &p = g.p[i];
+        const long mine = (long)p.N * (p.K / 8) * p.nb * p.M;
+        long want = budget * mine / (total_bytes > 0 ? total_bytes : 1);
+        if (want < 1) want = 1;
+        plan_problem(p, 1, want);
+        p.block_begin = begin;
+        begin += p.n_blocks;
+        any_split = any_split || p.ksplit > 1;
+    }
+    if (any_split) {
+        unsigned long long *base = nullptr;
+        int rc = get_workspace(stream, words, &base);
+        if (rc != LUTGEMM_OK) return rc;
+        size_t off = 0;
+        for (int i = 0; i < count; ++i) {
+            g.p[i].accum = base + off;
+            off += (size_t)g.p[i].M * g.p[i].N;
+        }
+    }
+    hipLaunchKernelGGL((lut_gemv_group_kernel<1>), dim3((unsigned)begin), dim3(kThreads), 0, stream, g);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return hip_fail(e);
+    return LUTGEMM_OK;
 }
 
 int lutgemm_gemv_uniform_f16(const uint32_t *bW, const void *alpha_f16, const void *qbias_f16,
@@ -655,8 +795,7 @@ int lutgemm_release_workspaces(void)
     std::lock_guard<std::mutex> lock(g_ws_mutex);
     for (auto it = g_workspaces.begin(); it != g_workspaces.end();) {
         if (it->first.first == dev) {
-            if (it->second.partial) (void)hipFree(it->second.partial);
-            if (it->second.tickets) (void)hipFree(it->second.tickets);
+            if (it->second.accum) (void)hipFree(it->second.accum);
             it = g_workspaces.erase(it);
         } else {
             ++it;

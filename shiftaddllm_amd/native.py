@@ -21,6 +21,7 @@ C_ABI_SYMBOLS = (
     "lutgemm_strerror",
     "lutgemm_last_hip_error",
     "lutgemm_gemv_rowwise_f16",
+    "lutgemm_gemv_rowwise_f16_grouped",
     "lutgemm_gemv_uniform_f16",
     "lutgemm_gemv_block_f16",
     "lutgemm_gemv_block_shift_u16",
@@ -29,6 +30,16 @@ C_ABI_SYMBOLS = (
     "lutgemm_copy_bytes",
     "lutgemm_release_workspaces",
 )
+
+
+MAX_GROUP = 8
+
+
+class RowwiseProblem(ctypes.Structure):
+    """struct lutgemm_rowwise_problem of include/lutgemm_gfx950.h."""
+    _fields_ = [("bW", ctypes.c_void_p), ("alpha_f16", ctypes.c_void_p), ("x_f16", ctypes.c_void_p),
+                ("out_f16", ctypes.c_void_p), ("N", ctypes.c_int), ("K", ctypes.c_int),
+                ("nb", ctypes.c_int), ("num_groups", ctypes.c_int), ("M", ctypes.c_int)]
 
 
 class NativeLibraryMissing(ImportError):
@@ -72,6 +83,8 @@ def cabi() -> ctypes.CDLL:
         lib.lutgemm_last_hip_error.argtypes = []
         lib.lutgemm_last_hip_error.restype = ci
         lib.lutgemm_gemv_rowwise_f16.argtypes = [vp, vp, vp, vp, ci, ci, ci, ci, ci, vp]
+        lib.lutgemm_gemv_rowwise_f16_grouped.argtypes = [ci, ctypes.POINTER(RowwiseProblem), vp]
+        lib.lutgemm_gemv_rowwise_f16_grouped.restype = ci
         lib.lutgemm_gemv_uniform_f16.argtypes = [vp, vp, vp, vp, vp, ci, ci, ci, ci, ci, vp]
         lib.lutgemm_gemv_block_f16.argtypes = [vp, vp, vp, vp, ci, ci, ci, ci, ci, vp]
         lib.lutgemm_gemv_block_shift_u16.argtypes = [vp, vp, vp, vp, ci, ci, ci, ci, ci, ci, vp]

@@ -28,7 +28,7 @@ def _declared_functions():
 
 def test_header_declares_the_expected_entry_points():
     names = _declared_functions()
-    for want in ("lutgemm_gemv_rowwise_f16", "lutgemm_gemv_uniform_f16", "lutgemm_gemv_block_f16",
+    for want in ("lutgemm_gemv_rowwise_f16", "lutgemm_gemv_rowwise_f16_grouped", "lutgemm_gemv_uniform_f16", "lutgemm_gemv_block_f16",
                  "lutgemm_gemv_block_shift_u16", "lutgemm_gemv_block_apot_i8"):
         assert want in names
 

@@ -299,3 +299,83 @@ def test_runs_on_a_side_stream(gpu_device):
         got = run_rowwise(gpu_device, p.bW, p.alpha, p.x, p.num_groups)
     s.synchronize()
     _assert_close(got, want)
+
+
+# ---- several GEMVs in one launch ------------------------------------------------
+
+def _grouped(dev, problems, outs=None):
+    """problems: list of RowwiseProblem (CPU). Returns the list of device outputs."""
+    lib = native.cabi()
+    arr = (native.RowwiseProblem * len(problems))()
+    keep = []
+    d_outs = []
+    for i, p in enumerate(problems):
+        M = p.x.shape[0]
+        d = [p.bW.to(dev), p.alpha.to(dev), p.x.to(dev).contiguous(),
+             (torch.zeros((M, p.N), dtype=torch.float16) if outs is None else outs[i].clone()).to(dev)]
+        keep.append(d)
+        d_outs.append(d[3])
+        arr[i] = native.RowwiseProblem(d[0].data_ptr(), d[1].data_ptr(), d[2].data_ptr(), d[3].data_ptr(),
+                                       p.N, p.K, p.nb, p.num_groups, M)
+    _check(lib.lutgemm_gemv_rowwise_f16_grouped(len(problems), arr, _stream()))
+    torch.cuda.synchronize()
+    return d_outs
+
+
+def test_grouped_launch_mixed_shapes_and_bits(gpu_device):
+    specs = [(512, 1024, 3, 128, 1), (1024, 1024, 2, 128, 1), (260, 288, 4, 32, 2), (4096, 512, 3, 128, 1),
+             (128, 2048, 1, 64, 1)]
+    probs = [workload.make_rowwise_problem(N, K, nb=nb, group_size=gs, M=M, seed=40 + i, quantize=False)
+             for i, (N, K, nb, gs, M) in enumerate(specs)]
+    bias = [torch.randn((p.x.shape[0], p.N), generator=torch.Generator().manual_seed(i)).half()
+            for i, p in enumerate(probs)]
+    got = _grouped(gpu_device, probs, outs=bias)
+    for p, b, g in zip(probs, bias, got):
+        want, _ = orc.gemv_rowwise_c(p.bW.numpy(), p.alpha.numpy(), p.x.numpy(), p.num_groups, out=b.numpy())
+        _assert_close(g, want, (p.N, p.K, p.nb))
+        # identical, bit for bit, to the single-problem entry point
+        assert torch.equal(g, run_rowwise(gpu_device, p.bW, p.alpha, p.x, p.num_groups, out=b))
+
+
+def test_grouped_llama7b_block(gpu_device):
+    # the seven linears of one decoder block in a single launch
+    probs = [workload.make_rowwise_problem(N, K, nb=3, group_size=128, seed=60 + i, quantize=False)
+             for i, (_, N, K) in enumerate(workload.LLAMA2_7B_LINEARS)]
+    got = _grouped(gpu_device, probs)
+    for p, g in zip(probs, got):
+        want, _ = orc.gemv_rowwise_c(p.bW.numpy(), p.alpha.numpy(), p.x.numpy(), p.num_groups)
+        _assert_close(g, want, (p.N, p.K))
+
+
+def test_grouped_rejects_bad_counts(gpu_device):
+    lib = native.cabi()
+    arr = (native.RowwiseProblem * 1)()
+    assert lib.lutgemm_gemv_rowwise_f16_grouped(0, arr, None) == -1
+    assert lib.lutgemm_gemv_rowwise_f16_grouped(native.MAX_GROUP + 1, arr, None) == -1
+    assert lib.lutgemm_gemv_rowwise_f16_grouped(1, arr, None) == -1      # null operands inside
+
+
+def test_repeated_calls_leave_the_workspace_clean(gpu_device):
+    # K-split accumulators are cleared by whoever completes a sum: many calls in a
+    # row, of different shapes on one stream, must keep giving the same answer
+    a = workload.make_rowwise_problem(1024, 4096, nb=3, group_size=128, seed=70, quantize=False)
+    b = workload.make_rowwise_problem(2048, 2048, nb=2, group_size=128, seed=71, quantize=False)
+    wa, _ = orc.gemv_rowwise_c(a.bW.numpy(), a.alpha.numpy(), a.x.numpy(), a.num_groups)
+    wb, _ = orc.gemv_rowwise_c(b.bW.numpy(), b.alpha.numpy(), b.x.numpy(), b.num_groups)
+    first = run_rowwise(gpu_device, a.bW, a.alpha, a.x, a.num_groups)
+    for _ in range(5):
+        _assert_close(run_rowwise(gpu_device, b.bW, b.alpha, b.x, b.num_groups), wb)
+        again = run_rowwise(gpu_device, a.bW, a.alpha, a.x, a.num_groups)
+        _assert_close(again, wa)
+        assert torch.equal(again, first)
+
+
+def test_saturation_of_non_finite_partial_sums(gpu_device):
+    # a NaN / inf activation must not poison the K-split accumulators for later calls
+    p = workload.make_rowwise_problem(512, 4096, nb=3, group_size=128, seed=72, quantize=False)
+    want, _ = orc.gemv_rowwise_c(p.bW.numpy(), p.alpha.numpy(), p.x.numpy(), p.num_groups)
+    bad = p.x.clone()
+    bad[0, 5] = float("inf")
+    y_bad = run_rowwise(gpu_device, p.bW, p.alpha, bad, p.num_groups)
+    assert not torch.isfinite(y_bad).all()
+    _assert_close(run_rowwise(gpu_device, p.bW, p.alpha, p.x, p.num_groups), want)
