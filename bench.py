@@ -258,9 +258,13 @@ def main():
         for g in pool[:7]:
             run(g, sp)
     stream.synchronize()
-    parity["fused_equals_plain_bitwise"] = all(torch.equal(a, g.out) for a, g in zip(fused_out, pool[:7]))
-    if not parity["fused_equals_plain_bitwise"]:
-        raise SystemExit("fused launch disagrees with separate launches")
+    # (K is cut differently in a fused launch, so fp32 partial sums round differently:
+    # the two paths agree to fp16 rounding, not bit for bit)
+    worst = max(oracle.error_metrics(a.float().cpu().numpy(), g.out.float().cpu().numpy())[0]
+                for a, g in zip(fused_out, pool[:7]))
+    parity["fused_vs_plain_rel_l2"] = worst
+    if worst > 2e-4:
+        raise SystemExit(f"fused launch disagrees with separate launches: rel_l2={worst}")
 
     # ---- every shape alone: hot (one buffer, cache resident) and rotating (HBM) --------
     shape_table = None

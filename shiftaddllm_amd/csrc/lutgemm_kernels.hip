@@ -6,19 +6,25 @@
 // in the ShiftAddLLM checkout); the operand layouts are the reference's, the
 // execution scheme is not:
 //
-//  * A workgroup (256 threads = 4 waves) owns an N-tile of 128*NSTEPS outputs
+//  * A workgroup (512 threads = 8 waves) owns an N-tile of 256*NSTEPS outputs
 //    and a contiguous K-slice, processed in "sets" of 256 inputs = 8 sign
 //    words = 32 eight-input chunks.
-//  * Per set it builds 32 partial-sum tables of 256 fp32 entries in LDS
-//    (32 KiB).  Table t lives entirely in LDS bank t: entry i of table t is
-//    dword i*32 + t.  A half-wave is arranged so that its 32 lanes always
-//    look up 32 different tables, hence 32 different banks: no bank conflicts
-//    by construction, whatever the data-dependent indices are.
+//  * Per set it builds 32 partial-sum tables of 256 fp32 entries in LDS.
+//    Entry i of table t of buffer f sits at byte i*256 + 4*(t + 32*f): every
+//    table lives entirely in LDS bank t, and two buffers interleave in the same
+//    64 KiB so that the tables of set i+1 are built while set i is looked up
+//    (one barrier per set).  A half-wave is arranged so that its 32 lanes always
+//    look up 32 different tables, hence 32 different banks: no bank conflicts by
+//    construction, whatever the data-dependent indices are.
+//  * The 256-byte entry stride makes a look-up address "index byte in bits
+//    8..15, per-lane bank offset in bits 0..7", which ONE v_perm_b32 assembles
+//    from the sign word and a per-lane constant; a look-up costs that, the
+//    ds_read_b32 and one fma.
 //  * Lane l of a wave: q = l&3, kw = (l>>2)&7, h = l>>5.  The lane streams
 //    128-bit loads of sign word (set*8 + kw) for the 4 outputs of quad
-//    (h*4+q); rows of the sign matrix are read in 512-byte contiguous runs
-//    per workgroup.  At look-up step j the lane uses byte (j+q)&3 of its
-//    word, i.e. table kw*4 + ((j+q)&3) -- distinct over (kw, q).
+//    (h*4+q); rows of the sign matrix are read in 1 KiB contiguous runs per
+//    workgroup.  At look-up step j the lane uses byte (j+q)&3 of its word,
+//    i.e. table kw*4 + ((j+q)&3) -- distinct over (kw, q).
 //  * The loads of set i+1 are issued before the look-ups of set i, so the
 //    HBM latency of a workgroup's own stream hides behind its LDS work.
 //  * Accumulation is fp32; alphas are applied with one fma per look-up
@@ -48,11 +54,14 @@ namespace {
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
-constexpr int kThreads = 256;
+constexpr int kThreads = 512;
+constexpr int kWaves = kThreads / 64;
 constexpr int kSetWords = 8;               // sign words (of 32 inputs) per table set
 constexpr int kTables = 4 * kSetWords;     // 32 tables, one per LDS bank
 constexpr int kWaveCols = 32;              // outputs a wave covers per step
-constexpr int kStepCols = 4 * kWaveCols;   // outputs a workgroup covers per step
+constexpr int kStepCols = kWaves * kWaveCols;  // outputs a workgroup covers per step
+constexpr int kEntryStride = 64;           // dwords between consecutive entries of a table
+constexpr int kLutDwords = 256 * kEntryStride;  // 64 KiB: two interleaved table buffers
 constexpr int kMaxKSplit = 32;             // bounded by the fixed-point accumulator layout
 constexpr int kMaxGroup = LUTGEMM_MAX_GROUP;  // problems per grouped launch
 
@@ -84,6 +93,7 @@ struct Problem {
     int ksplit;
     int n_tiles;
     int group_words;     // row-wise / uniform: words per alpha group
+    int group_shift;     // log2(group_words) when it is a power of two, else -1
     int R;               // block modes: row groups
     int rows_per_group;  // block modes: N / R
     int nb;
@@ -147,42 +157,58 @@ struct SetOperands {
     u32x4 xraw;                 // 8 activations of the chunk this thread builds a table for
 };
 
+// Per-lane address parts that do not change from set to set.
+template <int NSTEPS>
+struct LaneCols {
+    uint32_t col4[NSTEPS];  // byte offset of the lane's output quad inside a row of sign words
+    uint32_t col2[NSTEPS];  // same, inside a row of fp16 alphas
+    int rgroup[NSTEPS];     // block modes: alpha row group of the quad
+};
+
 // Issue every global load of one table set for this lane.  Branch-free on
 // purpose: out-of-range rows and columns are clamped to valid addresses instead
 // of predicated, so the loads sit in straight-line code and the compiler can
-// keep the NEXT set's loads in flight (s_waitcnt vmcnt(n), n > 0) while the
+// keep later sets' loads in flight (s_waitcnt vmcnt(n), n > 0) while the
 // current set is consumed.  Clamped data is harmless: tables of inputs beyond K
-// are all zero, and outputs beyond N are never written.
+// are all zero, and outputs beyond N are never written.  Addresses are a
+// uniform 64-bit base plus a 32-bit per-lane offset.
 template <int NB, int NSTEPS, int MODE>
 __device__ __forceinline__ void load_set(SetOperands<NB, NSTEPS, MODE> &r, const Problem &p,
-                                         const __half *x, int set, int kw, int q, int n_lane, int tb)
+                                         const __half *x, int set, int kw, int q,
+                                         const LaneCols<NSTEPS> &lc, int tb)
 {
-    const int row = min(set * kSetWords + kw, p.kwords - 1);
+    const int kwc = min(kw, p.kwords - 1 - set * kSetWords);  // only the last set of K can clamp
+    const uint32_t row_bytes = (uint32_t)p.N * 4u;            // one bit plane of one sign word row
+    const char *wbase = (const char *)p.W + (size_t)set * kSetWords * NB * row_bytes;
+    const uint32_t wrow = (uint32_t)kwc * (NB * row_bytes);
+    [[maybe_unused]] const int row = set * kSetWords + kwc;
+    [[maybe_unused]] const int g = p.group_shift >= 0 ? (row >> p.group_shift) : (row / p.group_words);
 #pragma unroll
     for (int s = 0; s < NSTEPS; ++s) {
-        const int n = min(n_lane + s * kStepCols, p.N - 4);
 #pragma unroll
         for (int b = 0; b < NB; ++b) {
-            const u32x4 *src = (const u32x4 *)(p.W + ((size_t)row * NB + b) * p.N + n);
-            r.w[s][b] = __builtin_nontemporal_load(src);
+            const char *src = wbase + (size_t)b * row_bytes;
+            r.w[s][b] = __builtin_nontemporal_load((const u32x4 *)(src + (wrow + lc.col4[s])));
         }
         if constexpr (MODE == kRowF16) {
-            const int g = row / p.group_words;
+            const uint32_t arow = (uint32_t)g * (NB * (uint32_t)p.N * 2u);
 #pragma unroll
-            for (int b = 0; b < NB; ++b)
-                r.a_row[s][b] = *(const u32x2 *)((const __half *)p.alpha + ((size_t)g * NB + b) * p.N + n);
+            for (int b = 0; b < NB; ++b) {
+                const char *src = (const char *)p.alpha + (size_t)b * p.N * 2u;
+                r.a_row[s][b] = *(const u32x2 *)(src + (arow + lc.col2[s]));
+            }
         } else if constexpr (MODE == kUniformF16) {
-            const int g = row / p.group_words;
-            r.a_uni[s] = *(const u32x2 *)((const __half *)p.alpha + (size_t)g * p.N + n);
-            r.q_uni[s] = *(const u32x2 *)(p.qbias + (size_t)g * p.N + n);
+            const uint32_t arow = (uint32_t)g * ((uint32_t)p.N * 2u);
+            r.a_uni[s] = *(const u32x2 *)((const char *)p.alpha + (arow + lc.col2[s]));
+            r.q_uni[s] = *(const u32x2 *)((const char *)p.qbias + (arow + lc.col2[s]));
         } else {
-            const int rg = n / p.rows_per_group;
 #pragma unroll
             for (int b = 0; b < NB; ++b)
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
                     const int chunk = row * 4 + ((j + q) & 3);
-                    r.a_blk[s][b][j] = load_block_alpha<MODE>(p.alpha, ((size_t)chunk * NB + b) * p.R + rg);
+                    r.a_blk[s][b][j] =
+                        load_block_alpha<MODE>(p.alpha, ((size_t)chunk * NB + b) * p.R + lc.rgroup[s]);
                 }
         }
     }
@@ -195,64 +221,65 @@ __device__ __forceinline__ void load_set(SetOperands<NB, NSTEPS, MODE> &r, const
     r.xraw.w = live ? xr.w : 0u;
 }
 
-// Build the 32 tables of one set, then run this lane's look-ups against them.
-template <int NB, int NSTEPS, int MODE>
-__device__ __forceinline__ void consume_set(const SetOperands<NB, NSTEPS, MODE> &cur, float *lut,
-                                            float (&acc)[NSTEPS][4], const int (&bank)[4], int q,
-                                            int tb, int eb)
+// Build the 32 tables of one set into buffer `buf` (0/1).  Thread (tb, eb)
+// writes entries eb*16 .. eb*16+15 of table tb: bits 4..7 of the entry index
+// come from eb, bits 0..3 are walked in Gray-code order, one add per entry.
+__device__ __forceinline__ void build_tables(const u32x4 &xraw, float *lut, int buf, int tb, int eb)
 {
-    // ---- build: this thread writes entries eb*32 .. +31 of table tb -----------
     float x2[8];  // 2 * x
     float base = 0.0f;
-    {
-        const uint32_t r4[4] = {cur.xraw.x, cur.xraw.y, cur.xraw.z, cur.xraw.w};
+    const uint32_t r4[4] = {xraw.x, xraw.y, xraw.z, xraw.w};
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const float lo = half_bits_to_float(r4[j] & 0xffffu);
-            const float hi = half_bits_to_float(r4[j] >> 16);
-            x2[2 * j] = lo + lo;
-            x2[2 * j + 1] = hi + hi;
-            base -= lo + hi;  // entry 0 = -sum x
+    for (int j = 0; j < 4; ++j) {
+        const float lo = half_bits_to_float(r4[j] & 0xffffu);
+        const float hi = half_bits_to_float(r4[j] >> 16);
+        x2[2 * j] = lo + lo;
+        x2[2 * j + 1] = hi + hi;
+        base -= lo + hi;  // entry 0 = -sum x
+    }
+    float top = base;
+#pragma unroll
+    for (int j = 4; j < 8; ++j)
+        if ((eb >> (j - 4)) & 1) top += x2[j];
+    float *col = lut + (eb * 16) * kEntryStride + buf * kTables + tb;
+#pragma unroll
+    for (int sb = 0; sb < 2; ++sb) {  // bit 3 fixed per sub-block: two short chains
+        float v = top;
+        if (sb & 1) v += x2[3];
+        unsigned gray = 0;
+        col[(sb * 8) * kEntryStride] = v;
+#pragma unroll
+        for (int i = 1; i < 8; ++i) {
+            const int bit = __builtin_ctz(i);
+            gray ^= 1u << bit;
+            v += ((gray >> bit) & 1u) ? x2[bit] : -x2[bit];
+            col[(sb * 8 + gray) * kEntryStride] = v;
         }
     }
-    __syncthreads();  // look-ups of the previous set are done with the tables
-    {
-        float top = base;  // bits 5..7 of the entry index come from eb
-#pragma unroll
-        for (int j = 5; j < 8; ++j)
-            if ((eb >> (j - 5)) & 1) top += x2[j];
-        float *col = lut + (eb * 32) * kTables + tb;
-#pragma unroll
-        for (int sb = 0; sb < 4; ++sb) {  // bits 3,4 fixed per sub-block: 4 short chains
-            float v = top;
-            if (sb & 1) v += x2[3];
-            if (sb & 2) v += x2[4];
-            unsigned gray = 0;
-            col[(sb * 8) * kTables] = v;
-#pragma unroll
-            for (int i = 1; i < 8; ++i) {
-                const int bit = __builtin_ctz(i);
-                gray ^= 1u << bit;
-                v += ((gray >> bit) & 1u) ? x2[bit] : -x2[bit];
-                col[(sb * 8 + gray) * kTables] = v;
-            }
-        }
-    }
-    __syncthreads();
+}
 
-    // ---- look-ups, software pipelined in units of 16 (one bit plane of one step):
-    // the LDS reads of unit u+1 are issued before the fmas of unit u
+// This lane's look-ups of one set against table buffer `lane_off` selects.
+// lane_off: byte j = 4*(bank of the table used at step j + 32*buffer).
+// sel[j]  : v_perm_b32 selector putting byte (j+q)&3 of the sign word into
+//           bits 8..15 and byte j of lane_off into bits 0..7.
+// Software pipelined in units of 16 look-ups (one bit plane of one step): the
+// LDS reads of unit u+1 are issued before the fmas of unit u.
+template <int NB, int NSTEPS, int MODE>
+__device__ __forceinline__ void lookup_set(const SetOperands<NB, NSTEPS, MODE> &cur, const float *lut,
+                                           float (&acc)[NSTEPS][4], uint32_t lane_off,
+                                           const uint32_t (&sel)[4])
+{
+    const char *lut_bytes = (const char *)lut;
     constexpr int kUnits = NSTEPS * NB;
     float val[2][16];
     auto issue = [&](int u, float (&v)[16]) {
         const int s = u / NB, b = u % NB;
         const uint32_t w4[4] = {cur.w[s][b].x, cur.w[s][b].y, cur.w[s][b].z, cur.w[s][b].w};
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const uint32_t w = __builtin_rotateright32(w4[i], 8 * q);
+        for (int i = 0; i < 4; ++i)
 #pragma unroll
-            for (int j = 0; j < 4; ++j) v[4 * i + j] = lut[((w >> (8 * j)) & 255u) * kTables + bank[j]];
-        }
+            for (int j = 0; j < 4; ++j)
+                v[4 * i + j] = *(const float *)(lut_bytes + __builtin_amdgcn_perm(w4[i], lane_off, sel[j]));
     };
     auto retire = [&](int u, const float (&v)[16]) {
         const int s = u / NB, b = u % NB;
@@ -275,9 +302,11 @@ __device__ __forceinline__ void consume_set(const SetOperands<NB, NSTEPS, MODE> 
     };
     issue(0, val[0]);
     if constexpr (MODE == kUniformF16) {
+        // sum of the lane's 32 inputs = entry 255 of its four tables
         float sum_x = 0.0f;
 #pragma unroll
-        for (int j = 0; j < 4; ++j) sum_x += lut[255 * kTables + bank[j]];
+        for (int j = 0; j < 4; ++j)
+            sum_x += *(const float *)(lut_bytes + 255 * 4 * kEntryStride + ((lane_off >> (8 * j)) & 255u));
 #pragma unroll
         for (int s = 0; s < NSTEPS; ++s) {
             const uint32_t rq[2] = {cur.q_uni[s].x, cur.q_uni[s].y};
@@ -308,10 +337,15 @@ __device__ __forceinline__ void gemv_tile(const Problem &p, int tile, int kslice
 
     const __half *x = p.x + (size_t)m * p.K;
 
-    // dword offset of "my" table inside an entry row, per look-up step
-    int bank[4];
+    // per-lane look-up constants (see lookup_set)
+    uint32_t lane_off = 0;
+    uint32_t sel[4];
 #pragma unroll
-    for (int j = 0; j < 4; ++j) bank[j] = kw * 4 + ((j + q) & 3);
+    for (int j = 0; j < 4; ++j) {
+        const int jj = (j + q) & 3;
+        lane_off |= (uint32_t)(4 * (kw * 4 + jj)) << (8 * j);
+        sel[j] = 0x0c0c0000u | ((uint32_t)(4 + jj) << 8) | (uint32_t)j;
+    }
 
     float acc[NSTEPS][4];
 #pragma unroll
@@ -321,38 +355,60 @@ __device__ __forceinline__ void gemv_tile(const Problem &p, int tile, int kslice
 
     // table-build role of this thread
     const int tb = tid & 31;  // table (bank)
-    const int eb = tid >> 5;  // entries eb*32 .. eb*32+31
+    const int eb = tid >> 5;  // entries eb*16 .. eb*16+15
 
     const int set_begin = kslice * p.sets_per_split;
     const int set_end = min(set_begin + p.sets_per_split, p.nsets);
 
-    // two operand buffers used alternately, so that no register copy (which would
-    // have to wait for the loads) sits between a set's loads and its use
+    LaneCols<NSTEPS> lc;
+#pragma unroll
+    for (int s = 0; s < NSTEPS; ++s) {
+        const int n = min(n_lane + s * kStepCols, p.N - 4);
+        lc.col4[s] = (uint32_t)n * 4u;
+        lc.col2[s] = (uint32_t)n * 2u;
+        lc.rgroup[s] = (MODE == kBlockF16 || MODE == kBlockShiftU16 || MODE == kBlockApotI8)
+                           ? n / p.rows_per_group : 0;
+    }
+
+    // Two operand buffers used alternately: while set i is looked up, the loads of
+    // set i+1 are in flight.  No register copies between them (a copy would have
+    // to wait for the loads), and the has-next test is peeled out of the load
+    // path so that the compiler can count the loads in flight exactly.
     SetOperands<NB, NSTEPS, MODE> opA, opB;
-    load_set<NB, NSTEPS, MODE>(opA, p, x, set_begin, kw, q, n_lane, tb);
+    load_set<NB, NSTEPS, MODE>(opA, p, x, set_begin, kw, q, lc, tb);
 
     // the caller's output, needed only by whoever completes a sum: fetched now,
     // off the critical path
     u32x2 out_raw[NSTEPS];
     __half *out = p.out + (size_t)m * p.N;
 #pragma unroll
-    for (int s = 0; s < NSTEPS; ++s)
-        out_raw[s] = *(const u32x2 *)(out + min(n_lane + s * kStepCols, p.N - 4));
+    for (int s = 0; s < NSTEPS; ++s) out_raw[s] = *(const u32x2 *)((const char *)out + lc.col2[s]);
 
+    build_tables(opA.xraw, lut, 0, tb, eb);
+    __syncthreads();
+    // Steady state, per set: issue the loads of the next set, look the current
+    // set up in table buffer f, build the next set's tables into buffer f^1, one
+    // barrier.  The barrier both publishes buffer f^1 and retires the readers of
+    // buffer f, which the iteration after next overwrites.
+    constexpr uint32_t kFlip = 0x80808080u;  // +128 bytes = the other table buffer
     for (int set = set_begin;;) {
         if (set + 1 >= set_end) {
-            consume_set<NB, NSTEPS, MODE>(opA, lut, acc, bank, q, tb, eb);
+            lookup_set<NB, NSTEPS, MODE>(opA, lut, acc, lane_off, sel);
             break;
         }
-        load_set<NB, NSTEPS, MODE>(opB, p, x, set + 1, kw, q, n_lane, tb);
-        consume_set<NB, NSTEPS, MODE>(opA, lut, acc, bank, q, tb, eb);
+        load_set<NB, NSTEPS, MODE>(opB, p, x, set + 1, kw, q, lc, tb);
+        lookup_set<NB, NSTEPS, MODE>(opA, lut, acc, lane_off, sel);
+        build_tables(opB.xraw, lut, 1, tb, eb);
+        __syncthreads();
         ++set;
         if (set + 1 >= set_end) {
-            consume_set<NB, NSTEPS, MODE>(opB, lut, acc, bank, q, tb, eb);
+            lookup_set<NB, NSTEPS, MODE>(opB, lut, acc, lane_off ^ kFlip, sel);
             break;
         }
-        load_set<NB, NSTEPS, MODE>(opA, p, x, set + 1, kw, q, n_lane, tb);
-        consume_set<NB, NSTEPS, MODE>(opB, lut, acc, bank, q, tb, eb);
+        load_set<NB, NSTEPS, MODE>(opA, p, x, set + 1, kw, q, lc, tb);
+        lookup_set<NB, NSTEPS, MODE>(opB, lut, acc, lane_off ^ kFlip, sel);
+        build_tables(opA.xraw, lut, 0, tb, eb);
+        __syncthreads();
         ++set;
     }
 
@@ -429,7 +485,7 @@ __device__ __forceinline__ void gemv_tile(const Problem &p, int tile, int kslice
 template <int NB, int NSTEPS, int MODE>
 __global__ void __launch_bounds__(kThreads) lut_gemv_kernel(const Problem p)
 {
-    __shared__ __attribute__((aligned(16))) float lut[256 * kTables];
+    __shared__ __attribute__((aligned(16))) float lut[kLutDwords];
     int tile, kslice, m;
     decode_block(p, (int)blockIdx.x, tile, kslice, m);
     gemv_tile<NB, NSTEPS, MODE>(p, tile, kslice, m, lut);
@@ -440,7 +496,7 @@ __global__ void __launch_bounds__(kThreads) lut_gemv_kernel(const Problem p)
 template <int NSTEPS>
 __global__ void __launch_bounds__(kThreads) lut_gemv_group_kernel(const Group g)
 {
-    __shared__ __attribute__((aligned(16))) float lut[256 * kTables];
+    __shared__ __attribute__((aligned(16))) float lut[kLutDwords];
     const int b = blockIdx.x;
     int pi = 0;
 #pragma unroll
@@ -524,10 +580,11 @@ int env_int(const char *name, int fallback)
 }
 
 // Tuning knobs (read once): LUTGEMM_TARGET_BLOCKS = workgroups a launch aims
-// for, LUTGEMM_NSTEPS = 1 or 2 output steps per workgroup.
+// for (64 KiB of tables per workgroup lets two be resident per CU),
+// LUTGEMM_NSTEPS = 1 or 2 output steps per workgroup.
 int target_blocks()
 {
-    static const int v = env_int("LUTGEMM_TARGET_BLOCKS", 1024);
+    static const int v = env_int("LUTGEMM_TARGET_BLOCKS", 512);  // 2 workgroups x 256 CUs
     return v;
 }
 int forced_nsteps()
@@ -618,6 +675,9 @@ int fill_problem(Problem &p, int mode, const uint32_t *bW, const void *alpha, co
         const int gs = K / num_groups;
         if (gs % 32 != 0) return LUTGEMM_EINVAL;  // a sign word may not straddle two groups
         p.group_words = gs / 32;
+        p.group_shift = -1;
+        for (int sh = 0; sh < 20; ++sh)
+            if ((1 << sh) == p.group_words) p.group_shift = sh;
         if (!aligned(alpha, 8)) return LUTGEMM_EALIGN;
         if (mode == kUniformF16 && !aligned(qbias, 8)) return LUTGEMM_EALIGN;
     } else {

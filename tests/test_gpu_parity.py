@@ -333,8 +333,11 @@ def test_grouped_launch_mixed_shapes_and_bits(gpu_device):
     for p, b, g in zip(probs, bias, got):
         want, _ = orc.gemv_rowwise_c(p.bW.numpy(), p.alpha.numpy(), p.x.numpy(), p.num_groups, out=b.numpy())
         _assert_close(g, want, (p.N, p.K, p.nb))
-        # identical, bit for bit, to the single-problem entry point
-        assert torch.equal(g, run_rowwise(gpu_device, p.bW, p.alpha, p.x, p.num_groups, out=b))
+        # agrees with the single-problem entry point to fp16 rounding (K may be cut
+        # differently, so the fp32 partial sums are not bit-identical)
+        single = run_rowwise(gpu_device, p.bW, p.alpha, p.x, p.num_groups, out=b)
+        rel, _ = orc.error_metrics(g.float().cpu().numpy(), single.float().cpu().numpy())
+        assert rel <= 2e-4
 
 
 def test_grouped_llama7b_block(gpu_device):
