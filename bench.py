@@ -46,6 +46,8 @@ def parse_args():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying a HIP graph")
     ap.add_argument("--no-shape-table", action="store_true", help="skip timing every shape alone")
+    ap.add_argument("--plain-only", action="store_true",
+                    help="only the 224-launch step (no fused sequences, no per-shape table): for profiler runs")
     ap.add_argument("--profile-shape", type=str, default="",
                     help="N,K[,nb[,iters]]: only launch this shape repeatedly (for rocprofv3 runs) and exit")
     ap.add_argument("--profile-copy", type=int, default=0,
@@ -148,9 +150,10 @@ def main():
     import numpy as np
     import oracle
     parity = {}
+    torch.cuda.synchronize()                  # pool tensors were made on the default stream
     for g in pool[3:7]:                       # o_proj, gate, up, down of block 0
-        g.out.zero_()
         with torch.cuda.stream(stream):
+            g.out.zero_()
             run(g, sp)
         stream.synchronize()
         want, _ = oracle.gemv_rowwise_c(g.bW.cpu().numpy(), g.alpha.cpu().numpy(), g.x.cpu().numpy(), g.groups)
@@ -234,8 +237,9 @@ def main():
 
     # ---- the same step with fused launches --------------------------------------------
     fused = {}
-    for label, groups, launches in (("fused_qkv_o_gateup_down", fused4, 4 * len(blocks)),
-                                    ("fused_7_in_1", fused1, len(blocks))):
+    for label, groups, launches in (() if args.plain_only else
+                                    (("fused_qkv_o_gateup_down", fused4, 4 * len(blocks)),
+                                     ("fused_7_in_1", fused1, len(blocks)))):
         f = seq_fused(groups)
         gr = capture(f)
         _, dms = timed(f, gr, args.steps, args.warmup)
@@ -246,29 +250,28 @@ def main():
                         "achieved_GBps": round(gbs, 1), "frac_hbm_peak": round(gbs / HBM_PEAK_GBS, 4),
                         "decode_tokens_per_s_linears_only": round(1e3 / dms, 1)}
     # parity of the fused path (outputs accumulate: clear, run once, compare with a plain call)
-    for g in pool[:7]:
-        g.out.zero_()
-    with torch.cuda.stream(stream):
-        run_group(fused1[0][0])
-    stream.synchronize()
-    fused_out = [g.out.clone() for g in pool[:7]]
-    for g in pool[:7]:
-        g.out.zero_()
-    with torch.cuda.stream(stream):
-        for g in pool[:7]:
-            run(g, sp)
-    stream.synchronize()
-    # (K is cut differently in a fused launch, so fp32 partial sums round differently:
-    # the two paths agree to fp16 rounding, not bit for bit)
-    worst = max(oracle.error_metrics(a.float().cpu().numpy(), g.out.float().cpu().numpy())[0]
-                for a, g in zip(fused_out, pool[:7]))
-    parity["fused_vs_plain_rel_l2"] = worst
-    if worst > 2e-4:
-        raise SystemExit(f"fused launch disagrees with separate launches: rel_l2={worst}")
+    if not args.plain_only:
+        with torch.cuda.stream(stream):
+            for g in pool[:7]:
+                g.out.zero_()
+            run_group(fused1[0][0])
+            fused_out = [g.out.clone() for g in pool[:7]]
+            for g in pool[:7]:
+                g.out.zero_()
+            for g in pool[:7]:
+                run(g, sp)
+        stream.synchronize()
+        # (K is cut differently in a fused launch, so fp32 partial sums round differently:
+        # the two paths agree to fp16 rounding, not bit for bit)
+        worst = max(oracle.error_metrics(a.float().cpu().numpy(), g.out.float().cpu().numpy())[0]
+                    for a, g in zip(fused_out, pool[:7]))
+        parity["fused_vs_plain_rel_l2"] = worst
+        if worst > 2e-4:
+            raise SystemExit(f"fused launch disagrees with separate launches: rel_l2={worst}")
 
     # ---- every shape alone: hot (one buffer, cache resident) and rotating (HBM) --------
     shape_table = None
-    if not args.no_shape_table:
+    if not (args.no_shape_table or args.plain_only):
         shape_table = {}
         for (N, K) in ((4096, 4096), (11008, 4096), (4096, 11008)):
             same = [g for g in pool if (g.N, g.K) == (N, K)]
@@ -339,7 +342,7 @@ def main():
         "decode_tokens_per_s_linears_only": round(1e3 / dev_ms_per_step, 1),
         "roofline": {"bound": "hbm", "achieved": round(achieved_gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved_gbs / HBM_PEAK_GBS, 4), "traffic": traffic,
-                     "kernel": "lut_gemv_kernel<3,2,row-wise>",
+                     "kernel": "lut_gemv_kernel<3, 1, 0> (nb=3, row-wise alpha)",
                      "algorithmic_bytes_per_launch": round(mean_bytes),
                      "avg_launch_us": round(us_per_call, 4)},
         "cpu_baseline": cpu,
