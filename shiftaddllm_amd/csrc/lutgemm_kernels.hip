@@ -45,6 +45,7 @@
 
 #include <map>
 #include <mutex>
+#include <type_traits>
 #include <utility>
 
 #include "lutgemm_gfx950.h"
@@ -98,6 +99,7 @@ struct Problem {
     int rows_per_group;  // block modes: N / R
     int nb;
     int block_begin;     // grouped launches: first flat workgroup index of this problem
+    int mchunks;         // activation rows are handled in chunks of MROWS
     int n_blocks;        // workgroups of this problem in the flat grid
 };
 
@@ -107,7 +109,7 @@ __device__ __forceinline__ void decode_block(const Problem &p, int local, int &t
     tile = local % p.n_tiles;
     local /= p.n_tiles;
     kslice = local % p.ksplit;
-    m = local / p.ksplit;
+    m = local / p.ksplit;  // row chunk
 }
 
 struct Group {
@@ -154,7 +156,6 @@ struct SetOperands {
     float a_blk[NSTEPS][NB][4]; // block: one multiplier per look-up step
     u32x2 a_uni[NSTEPS];        // uniform: alpha per output
     u32x2 q_uni[NSTEPS];        // uniform: q_bias per output
-    u32x4 xraw;                 // 8 activations of the chunk this thread builds a table for
 };
 
 // Per-lane address parts that do not change from set to set.
@@ -173,9 +174,8 @@ struct LaneCols {
 // are all zero, and outputs beyond N are never written.  Addresses are a
 // uniform 64-bit base plus a 32-bit per-lane offset.
 template <int NB, int NSTEPS, int MODE>
-__device__ __forceinline__ void load_set(SetOperands<NB, NSTEPS, MODE> &r, const Problem &p,
-                                         const __half *x, int set, int kw, int q,
-                                         const LaneCols<NSTEPS> &lc, int tb)
+__device__ __forceinline__ void load_set(SetOperands<NB, NSTEPS, MODE> &r, const Problem &p, int set,
+                                         int kw, int q, const LaneCols<NSTEPS> &lc)
 {
     const int kwc = min(kw, p.kwords - 1 - set * kSetWords);  // only the last set of K can clamp
     const uint32_t row_bytes = (uint32_t)p.N * 4u;            // one bit plane of one sign word row
@@ -212,13 +212,21 @@ __device__ __forceinline__ void load_set(SetOperands<NB, NSTEPS, MODE> &r, const
                 }
         }
     }
+}
+
+// The 8 activations (fp16) of the chunk whose table this thread helps to build:
+// chunk tb of set `set` of activation row x.  Chunks beyond K read as zero.
+__device__ __forceinline__ u32x4 load_x_chunk(const Problem &p, const __half *x, int set, int tb)
+{
     const int k0 = (set * kTables + tb) * 8;
     const u32x4 xr = *(const u32x4 *)(x + min(k0, p.K - 8));
     const bool live = k0 < p.K;
-    r.xraw.x = live ? xr.x : 0u;
-    r.xraw.y = live ? xr.y : 0u;
-    r.xraw.z = live ? xr.z : 0u;
-    r.xraw.w = live ? xr.w : 0u;
+    u32x4 r;
+    r.x = live ? xr.x : 0u;
+    r.y = live ? xr.y : 0u;
+    r.z = live ? xr.z : 0u;
+    r.w = live ? xr.w : 0u;
+    return r;
 }
 
 // Build the 32 tables of one set into buffer `buf` (0/1).  Thread (tb, eb)
@@ -322,9 +330,12 @@ __device__ __forceinline__ void lookup_set(const SetOperands<NB, NSTEPS, MODE> &
     }
 }
 
-// One workgroup's share: N-tile `tile`, K-slice `kslice`, activation row `m`.
-template <int NB, int NSTEPS, int MODE>
-__device__ __forceinline__ void gemv_tile(const Problem &p, int tile, int kslice, int m, float *lut)
+// One workgroup's share: N-tile `tile`, K-slice `kslice`, activation rows
+// mchunk*MROWS .. +MROWS-1.  The sign words of a set are loaded once and used
+// for all MROWS rows; tables are built per (set, row) and double buffered, so the
+// work items of the pipeline are the (set, row) pairs in order.
+template <int NB, int NSTEPS, int MODE, int MROWS>
+__device__ __forceinline__ void gemv_tile(const Problem &p, int tile, int kslice, int mchunk, float *lut)
 {
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -334,8 +345,12 @@ __device__ __forceinline__ void gemv_tile(const Problem &p, int tile, int kslice
     const int h = lane >> 5;
     const int tile0 = tile * (kStepCols * NSTEPS);
     const int n_lane = tile0 + wave * kWaveCols + (h * 4 + q) * 4;  // + s*kStepCols
+    const int m0 = mchunk * MROWS;
 
-    const __half *x = p.x + (size_t)m * p.K;
+    // rows beyond M are clamped to the last row (computed twice, written once)
+    const __half *xrow[MROWS];
+#pragma unroll
+    for (int r = 0; r < MROWS; ++r) xrow[r] = p.x + (size_t)min(m0 + r, p.M - 1) * p.K;
 
     // per-lane look-up constants (see lookup_set)
     uint32_t lane_off = 0;
@@ -347,11 +362,13 @@ __device__ __forceinline__ void gemv_tile(const Problem &p, int tile, int kslice
         sel[j] = 0x0c0c0000u | ((uint32_t)(4 + jj) << 8) | (uint32_t)j;
     }
 
-    float acc[NSTEPS][4];
+    float acc[MROWS][NSTEPS][4];
 #pragma unroll
-    for (int s = 0; s < NSTEPS; ++s)
+    for (int r = 0; r < MROWS; ++r)
 #pragma unroll
-        for (int i = 0; i < 4; ++i) acc[s][i] = 0.0f;
+        for (int s = 0; s < NSTEPS; ++s)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) acc[r][s][i] = 0.0f;
 
     // table-build role of this thread
     const int tb = tid & 31;  // table (bank)
@@ -375,120 +392,147 @@ __device__ __forceinline__ void gemv_tile(const Problem &p, int tile, int kslice
     // to wait for the loads), and the has-next test is peeled out of the load
     // path so that the compiler can count the loads in flight exactly.
     SetOperands<NB, NSTEPS, MODE> opA, opB;
-    load_set<NB, NSTEPS, MODE>(opA, p, x, set_begin, kw, q, lc, tb);
+    load_set<NB, NSTEPS, MODE>(opA, p, set_begin, kw, q, lc);
 
     // the caller's output, needed only by whoever completes a sum: fetched now,
     // off the critical path
-    u32x2 out_raw[NSTEPS];
-    __half *out = p.out + (size_t)m * p.N;
+    u32x2 out_raw[MROWS][NSTEPS];
 #pragma unroll
-    for (int s = 0; s < NSTEPS; ++s) out_raw[s] = *(const u32x2 *)((const char *)out + lc.col2[s]);
+    for (int r = 0; r < MROWS; ++r)
+#pragma unroll
+        for (int s = 0; s < NSTEPS; ++s)
+            out_raw[r][s] = *(const u32x2 *)((const char *)(p.out + (size_t)min(m0 + r, p.M - 1) * p.N) + lc.col2[s]);
 
-    build_tables(opA.xraw, lut, 0, tb, eb);
+    int buf = 0;
+    build_tables(load_x_chunk(p, xrow[0], set_begin, tb), lut, 0, tb, eb);
     __syncthreads();
-    // Steady state, per set: issue the loads of the next set, look the current
-    // set up in table buffer f, build the next set's tables into buffer f^1, one
-    // barrier.  The barrier both publishes buffer f^1 and retires the readers of
-    // buffer f, which the iteration after next overwrites.
+    // Steady state, per (set, row) item: fetch the activations of the next item,
+    // look the current item up in table buffer f, build the next item's tables into
+    // buffer f^1, one barrier.  The barrier both publishes buffer f^1 and retires
+    // the readers of buffer f, which the item after next overwrites.
     constexpr uint32_t kFlip = 0x80808080u;  // +128 bytes = the other table buffer
+    auto rows_of_set = [&](const SetOperands<NB, NSTEPS, MODE> &ops, int set, auto has_next_set) {
+#pragma unroll
+        for (int r = 0; r < MROWS; ++r) {
+            const bool more = (r + 1 < MROWS) || decltype(has_next_set)::value;
+            u32x4 xn = (u32x4){0u, 0u, 0u, 0u};
+            if (more)
+                xn = (r + 1 < MROWS) ? load_x_chunk(p, xrow[(r + 1) % MROWS], set, tb)
+                                     : load_x_chunk(p, xrow[0], set + 1, tb);
+            // opaque to the optimiser: otherwise the 48 look-up addresses of a set are
+            // kept in registers across all rows instead of being recomputed (1 op each)
+            asm volatile("" : "+v"(lane_off));
+            lookup_set<NB, NSTEPS, MODE>(ops, lut, acc[r], lane_off, sel);
+            if (more) {
+                buf ^= 1;
+                lane_off ^= kFlip;
+                build_tables(xn, lut, buf, tb, eb);
+                __syncthreads();
+            }
+        }
+    };
     for (int set = set_begin;;) {
         if (set + 1 >= set_end) {
-            lookup_set<NB, NSTEPS, MODE>(opA, lut, acc, lane_off, sel);
+            rows_of_set(opA, set, std::false_type{});
             break;
         }
-        load_set<NB, NSTEPS, MODE>(opB, p, x, set + 1, kw, q, lc, tb);
-        lookup_set<NB, NSTEPS, MODE>(opA, lut, acc, lane_off, sel);
-        build_tables(opB.xraw, lut, 1, tb, eb);
-        __syncthreads();
+        load_set<NB, NSTEPS, MODE>(opB, p, set + 1, kw, q, lc);
+        rows_of_set(opA, set, std::true_type{});
         ++set;
         if (set + 1 >= set_end) {
-            lookup_set<NB, NSTEPS, MODE>(opB, lut, acc, lane_off ^ kFlip, sel);
+            rows_of_set(opB, set, std::false_type{});
             break;
         }
-        load_set<NB, NSTEPS, MODE>(opA, p, x, set + 1, kw, q, lc, tb);
-        lookup_set<NB, NSTEPS, MODE>(opB, lut, acc, lane_off ^ kFlip, sel);
-        build_tables(opA.xraw, lut, 0, tb, eb);
-        __syncthreads();
+        load_set<NB, NSTEPS, MODE>(opA, p, set + 1, kw, q, lc);
+        rows_of_set(opB, set, std::true_type{});
         ++set;
     }
 
     // ---- reduce the 8 kw-lanes of each output --------------------------------
 #pragma unroll
-    for (int s = 0; s < NSTEPS; ++s)
+    for (int r = 0; r < MROWS; ++r)
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            float v = acc[s][i];
-            v += __shfl_xor(v, 4);
-            v += __shfl_xor(v, 8);
-            v += __shfl_xor(v, 16);
-            acc[s][i] = v;
-        }
+        for (int s = 0; s < NSTEPS; ++s)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                float v = acc[r][s][i];
+                v += __shfl_xor(v, 4);
+                v += __shfl_xor(v, 8);
+                v += __shfl_xor(v, 16);
+                acc[r][s][i] = v;
+            }
     if (kw != 0) return;
 
-    if (p.ksplit == 1) {
+#pragma unroll
+    for (int r = 0; r < MROWS; ++r) {
+        const int m = m0 + r;
+        if (m >= p.M) break;
+        __half *out = p.out + (size_t)m * p.N;
+        if (p.ksplit == 1) {
+#pragma unroll
+            for (int s = 0; s < NSTEPS; ++s) {
+                const int n = n_lane + s * kStepCols;
+                if (n < p.N) {
+                    u32x2 raw = out_raw[r][s];
+                    const float o0 = half_bits_to_float(raw.x & 0xffffu) + acc[r][s][0];
+                    const float o1 = half_bits_to_float(raw.x >> 16) + acc[r][s][1];
+                    const float o2 = half_bits_to_float(raw.y & 0xffffu) + acc[r][s][2];
+                    const float o3 = half_bits_to_float(raw.y >> 16) + acc[r][s][3];
+                    raw.x = float_to_half_bits(o0) | (float_to_half_bits(o1) << 16);
+                    raw.y = float_to_half_bits(o2) | (float_to_half_bits(o3) << 16);
+                    *(u32x2 *)(out + n) = raw;
+                }
+            }
+            continue;
+        }
+
+        // ---- K-split: one returning fixed-point atomic per output ---------------
+        unsigned long long *accum = p.accum + (size_t)m * p.N;
+        unsigned long long contrib[NSTEPS][4], old[NSTEPS][4];
 #pragma unroll
         for (int s = 0; s < NSTEPS; ++s) {
             const int n = n_lane + s * kStepCols;
-            if (n < p.N) {
-                u32x2 raw = out_raw[s];
-                const float o0 = half_bits_to_float(raw.x & 0xffffu) + acc[s][0];
-                const float o1 = half_bits_to_float(raw.x >> 16) + acc[s][1];
-                const float o2 = half_bits_to_float(raw.y & 0xffffu) + acc[s][2];
-                const float o3 = half_bits_to_float(raw.y >> 16) + acc[s][3];
-                raw.x = float_to_half_bits(o0) | (float_to_half_bits(o1) << 16);
-                raw.y = float_to_half_bits(o2) | (float_to_half_bits(o3) << 16);
-                *(u32x2 *)(out + n) = raw;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                // non-finite or out-of-range partial sums saturate (fp16 rounds them to inf)
+                float v = acc[r][s][i];
+                v = (v == v) ? v : 65536.0f;
+                v = fminf(fmaxf(v, -65536.0f), 65536.0f);
+                const long long fx = __double2ll_rn((double)v * 4294967296.0);
+                contrib[s][i] = (unsigned long long)(fx + kBias) + kCountOne;
+                old[s][i] = 0;
+                if (n < p.N)
+                    old[s][i] = __hip_atomic_fetch_add(accum + n + i, contrib[s][i], __ATOMIC_RELAXED,
+                                                       __HIP_MEMORY_SCOPE_AGENT);
             }
         }
-        return;
-    }
-
-    // ---- K-split: one returning fixed-point atomic per output -------------------
-    unsigned long long *accum = p.accum + (size_t)m * p.N;
-    unsigned long long contrib[NSTEPS][4], old[NSTEPS][4];
 #pragma unroll
-    for (int s = 0; s < NSTEPS; ++s) {
-        const int n = n_lane + s * kStepCols;
+        for (int s = 0; s < NSTEPS; ++s) {
+            const int n = n_lane + s * kStepCols;
+            if (n >= p.N) continue;
+            const uint32_t raw2[2] = {out_raw[r][s].x, out_raw[r][s].y};
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            // non-finite or out-of-range partial sums saturate (fp16 rounds them to inf)
-            float v = acc[s][i];
-            v = (v == v) ? v : 65536.0f;
-            v = fminf(fmaxf(v, -65536.0f), 65536.0f);
-            const long long fx = __double2ll_rn((double)v * 4294967296.0);
-            contrib[s][i] = (unsigned long long)(fx + kBias) + kCountOne;
-            old[s][i] = 0;
-            if (n < p.N)
-                old[s][i] = __hip_atomic_fetch_add(accum + n + i, contrib[s][i], __ATOMIC_RELAXED,
-                                                   __HIP_MEMORY_SCOPE_AGENT);
-        }
-    }
-#pragma unroll
-    for (int s = 0; s < NSTEPS; ++s) {
-        const int n = n_lane + s * kStepCols;
-        if (n >= p.N) continue;
-        const uint32_t raw2[2] = {out_raw[s].x, out_raw[s].y};
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            if ((int)(old[s][i] >> 56) != p.ksplit - 1) continue;
-            // this contribution completed the sum
-            const long long total =
-                (long long)((old[s][i] + contrib[s][i]) & kSumMask) - (long long)p.ksplit * kBias;
-            const float y = (float)((double)total * (1.0 / 4294967296.0));
-            const float o = half_bits_to_float((raw2[i >> 1] >> (16 * (i & 1))) & 0xffffu) + y;
-            out[n + i] = __float2half_rn(o);
-            __hip_atomic_store(accum + n + i, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            for (int i = 0; i < 4; ++i) {
+                if ((int)(old[s][i] >> 56) != p.ksplit - 1) continue;
+                // this contribution completed the sum
+                const long long total =
+                    (long long)((old[s][i] + contrib[s][i]) & kSumMask) - (long long)p.ksplit * kBias;
+                const float y = (float)((double)total * (1.0 / 4294967296.0));
+                const float o = half_bits_to_float((raw2[i >> 1] >> (16 * (i & 1))) & 0xffffu) + y;
+                out[n + i] = __float2half_rn(o);
+                __hip_atomic_store(accum + n + i, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
         }
     }
 }
 
-template <int NB, int NSTEPS, int MODE>
+template <int NB, int NSTEPS, int MODE, int MROWS>
 __global__ void __launch_bounds__(kThreads) lut_gemv_kernel(const Problem p)
 {
     __shared__ __attribute__((aligned(16))) float lut[kLutDwords];
-    int tile, kslice, m;
-    decode_block(p, (int)blockIdx.x, tile, kslice, m);
-    gemv_tile<NB, NSTEPS, MODE>(p, tile, kslice, m, lut);
+    int tile, kslice, mchunk;
+    decode_block(p, (int)blockIdx.x, tile, kslice, mchunk);
+    gemv_tile<NB, NSTEPS, MODE, MROWS>(p, tile, kslice, mchunk, lut);
 }
 
 // Several row-wise problems in one launch (flat 1-D grid).  Bit widths may
@@ -506,10 +550,10 @@ __global__ void __launch_bounds__(kThreads) lut_gemv_group_kernel(const Group g)
     int tile, kslice, m;
     decode_block(p, b - p.block_begin, tile, kslice, m);
     switch (p.nb) {
-    case 1: gemv_tile<1, NSTEPS, kRowF16>(p, tile, kslice, m, lut); break;
-    case 2: gemv_tile<2, NSTEPS, kRowF16>(p, tile, kslice, m, lut); break;
-    case 3: gemv_tile<3, NSTEPS, kRowF16>(p, tile, kslice, m, lut); break;
-    default: gemv_tile<4, NSTEPS, kRowF16>(p, tile, kslice, m, lut); break;
+    case 1: gemv_tile<1, NSTEPS, kRowF16, 1>(p, tile, kslice, m, lut); break;
+    case 2: gemv_tile<2, NSTEPS, kRowF16, 1>(p, tile, kslice, m, lut); break;
+    case 3: gemv_tile<3, NSTEPS, kRowF16, 1>(p, tile, kslice, m, lut); break;
+    default: gemv_tile<4, NSTEPS, kRowF16, 1>(p, tile, kslice, m, lut); break;
     }
 }
 
@@ -595,16 +639,17 @@ int forced_nsteps()
 
 // Pick the N-tile and the K-split so that `want_blocks` workgroups exist while
 // each still does enough look-ups per table built.
-void plan_problem(Problem &p, int nsteps, long want_blocks)
+void plan_problem(Problem &p, int nsteps, int mrows, long want_blocks)
 {
     p.n_tiles = (p.N + kStepCols * nsteps - 1) / (kStepCols * nsteps);
-    long want = want_blocks / ((long)p.n_tiles * p.M);
+    p.mchunks = (p.M + mrows - 1) / mrows;
+    long want = want_blocks / ((long)p.n_tiles * p.mchunks);
     if (want < 1) want = 1;
     if (want > p.nsets) want = p.nsets;
     if (want > kMaxKSplit) want = kMaxKSplit;
     p.sets_per_split = (p.nsets + (int)want - 1) / (int)want;
     p.ksplit = (p.nsets + p.sets_per_split - 1) / p.sets_per_split;
-    p.n_blocks = p.n_tiles * p.ksplit * p.M;
+    p.n_blocks = p.n_tiles * p.ksplit * p.mchunks;
 }
 
 int pick_nsteps(int N)
@@ -618,28 +663,34 @@ int pick_nsteps(int N)
     return 1;
 }
 
+int pick_mrows(int M) { return M >= 3 ? 4 : M; }
+
 template <int NB, int MODE>
-int launch_nb(const Problem &p, int nsteps, hipStream_t stream)
+int launch_nb(const Problem &p, int nsteps, int mrows, hipStream_t stream)
 {
     dim3 grid((unsigned)p.n_blocks);
     dim3 block(kThreads);
-    if (nsteps == 1)
-        hipLaunchKernelGGL((lut_gemv_kernel<NB, 1, MODE>), grid, block, 0, stream, p);
+    if (mrows == 4)
+        hipLaunchKernelGGL((lut_gemv_kernel<NB, 1, MODE, 4>), grid, block, 0, stream, p);
+    else if (mrows == 2)
+        hipLaunchKernelGGL((lut_gemv_kernel<NB, 1, MODE, 2>), grid, block, 0, stream, p);
+    else if (nsteps == 1)
+        hipLaunchKernelGGL((lut_gemv_kernel<NB, 1, MODE, 1>), grid, block, 0, stream, p);
     else
-        hipLaunchKernelGGL((lut_gemv_kernel<NB, 2, MODE>), grid, block, 0, stream, p);
+        hipLaunchKernelGGL((lut_gemv_kernel<NB, 2, MODE, 1>), grid, block, 0, stream, p);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return hip_fail(e);
     return LUTGEMM_OK;
 }
 
 template <int MODE>
-int launch_mode(const Problem &p, int nsteps, hipStream_t stream)
+int launch_mode(const Problem &p, int nsteps, int mrows, hipStream_t stream)
 {
     switch (p.nb) {
-    case 1: return launch_nb<1, MODE>(p, nsteps, stream);
-    case 2: return launch_nb<2, MODE>(p, nsteps, stream);
-    case 3: return launch_nb<3, MODE>(p, nsteps, stream);
-    case 4: return launch_nb<4, MODE>(p, nsteps, stream);
+    case 1: return launch_nb<1, MODE>(p, nsteps, mrows, stream);
+    case 2: return launch_nb<2, MODE>(p, nsteps, mrows, stream);
+    case 3: return launch_nb<3, MODE>(p, nsteps, mrows, stream);
+    case 4: return launch_nb<4, MODE>(p, nsteps, mrows, stream);
     default: return LUTGEMM_EINVAL;
     }
 }
@@ -696,18 +747,19 @@ int run(int mode, const uint32_t *bW, const void *alpha, const void *qbias, cons
     int rc = fill_problem(p, mode, bW, alpha, qbias, x, out, N, K, nb, num_groups, M);
     if (rc != LUTGEMM_OK) return rc;
     hipStream_t stream = (hipStream_t)stream_v;
-    const int nsteps = pick_nsteps(N);
-    plan_problem(p, nsteps, target_blocks());
+    const int mrows = pick_mrows(M);
+    const int nsteps = mrows > 1 ? 1 : pick_nsteps(N);
+    plan_problem(p, nsteps, mrows, target_blocks());
     if (p.ksplit > 1) {
         rc = get_workspace(stream, (size_t)M * N, &p.accum);
         if (rc != LUTGEMM_OK) return rc;
     }
     switch (mode) {
-    case kRowF16: return launch_mode<kRowF16>(p, nsteps, stream);
-    case kBlockF16: return launch_mode<kBlockF16>(p, nsteps, stream);
-    case kBlockShiftU16: return launch_mode<kBlockShiftU16>(p, nsteps, stream);
-    case kBlockApotI8: return launch_mode<kBlockApotI8>(p, nsteps, stream);
-    case kUniformF16: return launch_mode<kUniformF16>(p, nsteps, stream);
+    case kRowF16: return launch_mode<kRowF16>(p, nsteps, mrows, stream);
+    case kBlockF16: return launch_mode<kBlockF16>(p, nsteps, mrows, stream);
+    case kBlockShiftU16: return launch_mode<kBlockShiftU16>(p, nsteps, mrows, stream);
+    case kBlockApotI8: return launch_mode<kBlockApotI8>(p, nsteps, mrows, stream);
+    case kUniformF16: return launch_mode<kUniformF16>(p, nsteps, mrows, stream);
     default: return LUTGEMM_EINVAL;
     }
 }
@@ -766,7 +818,7 @@ int lutgemm_gemv_rowwise_f16_grouped(int count, const lutgemm_rowwise_problem *p
         const long mine = (long)p.N * (p.K / 8) * p.nb * p.M;
         long want = budget * mine / (total_bytes > 0 ? total_bytes : 1);
         if (want < 1) want = 1;
-        plan_problem(p, 1, want);
+        plan_problem(p, 1, 1, want);
         p.block_begin = begin;
         begin += p.n_blocks;
         any_split = any_split || p.ksplit > 1;
