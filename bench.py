@@ -45,6 +45,7 @@ def parse_args():
     ap.add_argument("--layers", type=int, default=N_LAYERS, help="distinct decoder blocks in the weight pool")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying a HIP graph")
+    ap.add_argument("--no-decode", action="store_true", help="skip the full-model decode runs (config 4)")
     ap.add_argument("--no-shape-table", action="store_true", help="skip timing every shape alone")
     ap.add_argument("--plain-only", action="store_true",
                     help="only the 224-launch step (no fused sequences, no per-shape table): for profiler runs")
@@ -311,6 +312,40 @@ def main():
                "sample": f"one decoder block (7 GEMVs of this workload), weights dequantised once, fp32 "
                          f"torch linear, median of {len(samples)} passes; host shows {os.cpu_count()} cpus"}
 
+    launch_mode = "eager" if graph is None else "hip-graph replay"
+    # ---- config 4: full random-init Llama-2-7B decode, mixed 2/3/4-bit, batch 1 and 8 ----
+    decode_res = None
+    if not (args.no_decode or args.plain_only):
+        from shiftaddllm_amd import decode
+        launch_mode = "eager" if graph is None else "hip-graph replay"
+        del pool, blocks, fused4, fused1, graph
+        torch.cuda.empty_cache()
+        decode_res = {}
+        qc = workload.mixed_bit_config(decode.LLAMA2_7B.layers, seed=0)
+        counts = {b: sum(v["bits"] == b for v in qc.values()) for b in (2, 3, 4)}
+        for B in (1, 8):
+            model = decode.LutDecoder(decode.LLAMA2_7B, qc, batch=B, seed=0, device=dev, fuse_launches=True)
+            if not args.no_graph:
+                model.capture()
+            prompt = torch.randint(0, decode.LLAMA2_7B.vocab_size, (B, 128),
+                                   generator=torch.Generator().manual_seed(0))
+            r = decode.benchmark(model, prompt, generate=128, warmup=10)
+            lin_bytes = model.linear_bytes_per_token()
+            decode_res[f"batch{B}"] = {
+                "median_ms_per_token": round(r["median_s_per_token"] * 1e3, 4),
+                "tokens_per_s": round(r["tokens_per_s"], 1),
+                "median_ms_per_prompt_token": round(r["median_s_per_prompt_token"] * 1e3, 4),
+                "lut_gemm_algorithmic_GB_per_step": round(lin_bytes / 1e9, 3),
+                "lut_gemm_GBps_if_linears_were_all": round(lin_bytes / r["median_s_per_token"] / 1e9, 1),
+            }
+            del model
+            torch.cuda.empty_cache()
+        decode_res["config"] = ("random-init Llama-2-7B, 32 blocks, per-linear bits drawn 2:3:3:4 by "
+                                f"random.Random(0) ({counts[2]}x2-bit, {counts[3]}x3-bit, {counts[4]}x4-bit), "
+                                "group 128, fp16 RMSNorm/RoPE/attention in torch, 128 prompt tokens fed one by "
+                                "one then 128 greedy tokens, one HIP-graph replay + sync per token, "
+                                "q/k/v and gate/up as fused launches")
+
     traffic = None
     if os.path.exists(TRAFFIC_NOTE):
         for line in open(TRAFFIC_NOTE):
@@ -334,7 +369,7 @@ def main():
         "config": {"workload": "llama2-7b linears, 3-bit BCQ, group 128, pow2 alpha, batch 1: "
                                f"{args.layers} blocks x 7 GEMVs per step over distinct weights "
                                f"({step_bytes / 1e9:.3f} GB/step)",
-                   "launch": ("eager" if graph is None else "hip-graph replay") + ", one launch per GEMV",
+                   "launch": launch_mode + ", one launch per GEMV",
                    "calls_per_step": calls_per_step},
         "device_ms_per_step": round(dev_ms_per_step, 5),
         "achieved_GBps": round(achieved_gbs, 1),
@@ -347,6 +382,7 @@ def main():
                      "avg_launch_us": round(us_per_call, 4)},
         "cpu_baseline": cpu,
         "fused_launches": fused,
+        "decode": decode_res,
         "parity": parity,
         "pool_build_s": round(t_pool, 2),
     }

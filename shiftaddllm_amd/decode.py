@@ -1,0 +1,255 @@
+"""Token-by-token decode harness over LutLinear layers.
+
+Counterpart of the reference's kernel benchmark (`benchmark`, model/opt.py:367-423
+in the ShiftAddLLM checkout): warm-up single-token forwards, then every token --
+prompt tokens one at a time, then greedy continuations -- is one forward pass with
+a KV cache, followed by a device synchronisation and a wall-clock reading; the
+median seconds per token is reported.
+
+The reference drives a HuggingFace OPT with its linears swapped for LutLinear and
+needs the hub for the checkpoint.  This harness brings its own minimal
+Llama-architecture decoder (RMSNorm, rotary embeddings, grouped-query-capable
+attention over a static KV cache, SwiGLU MLP, fp16), random-initialised, whose
+seven linears per block are LutLinear modules with a per-linear bit width taken
+from a `{"<module>": {"bits": b, ...}}` map (the schema of the reference's
+--quant_config files, model/opt.py:83-88).  One decode step can be captured in a
+HIP graph; q/k/v and gate/up can be issued as one fused launch each.
+"""
+from __future__ import annotations
+
+import ctypes
+import math
+import statistics
+import time
+from dataclasses import dataclass
+
+import torch
+import torch.nn as nn
+import torch.nn.functional as F
+
+from . import native
+from .lut_gemm.quant import LutLinear
+
+
+@dataclass
+class DecoderConfig:
+    vocab_size: int = 32000
+    hidden: int = 4096
+    intermediate: int = 11008
+    layers: int = 32
+    heads: int = 32
+    kv_heads: int = 32
+    max_positions: int = 256
+    group_size: int = 128
+    rope_theta: float = 10000.0
+    rms_eps: float = 1e-5
+
+    @property
+    def head_dim(self):
+        return self.hidden // self.heads
+
+
+LLAMA2_7B = DecoderConfig()
+
+
+def random_lut_linear(in_f, out_f, bits, group_size, gen, device):
+    """LutLinear ("rowwise_fp16") with random sign planes and power-of-two scales
+    shaped like BCQ output of N(0, 0.02) weights: per (group, row) a base exponent,
+    one octave lower per further bit plane."""
+    lin = LutLinear(in_f, out_f, group_size=group_size, wbit=bits, bias=None, alpha_format="rowwise_fp16")
+    lin = lin.to(device)
+    lin.binaryWeight.data = torch.randint(-2 ** 31, 2 ** 31 - 1, (in_f // 32, bits, out_f), generator=gen,
+                                          device=device, dtype=torch.int32)
+    e = torch.randint(-8, -5, (in_f // group_size, 1, out_f), generator=gen, device=device).float()
+    e = e - torch.arange(bits, device=device).float().view(1, bits, 1)
+    lin.alpha.data = torch.exp2(e).to(torch.float16).contiguous()
+    return lin
+
+
+class Block(nn.Module):
+    def __init__(self, cfg: DecoderConfig, bits: dict, gen, device):
+        super().__init__()
+        h, kvd = cfg.hidden, cfg.kv_heads * cfg.head_dim
+        mk = lambda name, i, o: random_lut_linear(i, o, bits[name], cfg.group_size, gen, device)
+        self.q_proj = mk("self_attn.q_proj", h, h)
+        self.k_proj = mk("self_attn.k_proj", h, kvd)
+        self.v_proj = mk("self_attn.v_proj", h, kvd)
+        self.o_proj = mk("self_attn.o_proj", h, h)
+        self.gate_proj = mk("mlp.gate_proj", h, cfg.intermediate)
+        self.up_proj = mk("mlp.up_proj", h, cfg.intermediate)
+        self.down_proj = mk("mlp.down_proj", cfg.intermediate, h)
+        self.input_norm = nn.Parameter(torch.ones(h, dtype=torch.float16, device=device))
+        self.post_norm = nn.Parameter(torch.ones(h, dtype=torch.float16, device=device))
+
+
+def rms_norm(x, w, eps):
+    xf = x.float()
+    return (xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + eps)).to(x.dtype) * w
+
+
+class LutDecoder(nn.Module):
+    """Single-token-per-step decoder with a static KV cache of cfg.max_positions."""
+
+    def __init__(self, cfg: DecoderConfig, quant_config: dict | None = None, batch: int = 1, seed: int = 0,
+                 device="cuda:0", default_bits: int = 3, fuse_launches: bool = True,
+                 module_prefix: str = "model.layers"):
+        super().__init__()
+        self.cfg, self.batch, self.fuse = cfg, batch, fuse_launches
+        dev = torch.device(device)
+        gen = torch.Generator(device=dev).manual_seed(seed)
+        names = ("self_attn.q_proj", "self_attn.k_proj", "self_attn.v_proj", "self_attn.o_proj",
+                 "mlp.gate_proj", "mlp.up_proj", "mlp.down_proj")
+        self.blocks = nn.ModuleList()
+        for i in range(cfg.layers):
+            bits = {n: (quant_config or {}).get(f"{module_prefix}.{i}.{n}", {}).get("bits", default_bits)
+                    for n in names}
+            self.blocks.append(Block(cfg, bits, gen, dev))
+        scale = 0.02
+        self.embed = nn.Parameter((torch.randn((cfg.vocab_size, cfg.hidden), generator=gen, device=dev) * scale).half())
+        self.lm_head = nn.Parameter((torch.randn((cfg.vocab_size, cfg.hidden), generator=gen, device=dev) * scale).half())
+        self.final_norm = nn.Parameter(torch.ones(cfg.hidden, dtype=torch.float16, device=dev))
+        hd = cfg.head_dim
+        inv = 1.0 / (cfg.rope_theta ** (torch.arange(0, hd, 2, device=dev).float() / hd))
+        ang = torch.arange(cfg.max_positions, device=dev).float()[:, None] * inv[None, :]
+        self.register_buffer("cos", torch.cat([ang.cos(), ang.cos()], dim=-1).half(), persistent=False)
+        self.register_buffer("sin", torch.cat([ang.sin(), ang.sin()], dim=-1).half(), persistent=False)
+        shape = (cfg.layers, batch, cfg.kv_heads, cfg.max_positions, hd)
+        self.register_buffer("k_cache", torch.zeros(shape, dtype=torch.float16, device=dev), persistent=False)
+        self.register_buffer("v_cache", torch.zeros(shape, dtype=torch.float16, device=dev), persistent=False)
+        self.register_buffer("positions", torch.arange(cfg.max_positions, device=dev), persistent=False)
+        # static step inputs/outputs (graph replay reads and writes these)
+        self.register_buffer("ids", torch.zeros((batch,), dtype=torch.long, device=dev), persistent=False)
+        self.register_buffer("pos", torch.zeros((1,), dtype=torch.long, device=dev), persistent=False)
+        self.register_buffer("logits", torch.zeros((batch, cfg.vocab_size), dtype=torch.float16, device=dev),
+                             persistent=False)
+        self._graph = None
+        self._stream = None
+
+    # ---- linear layers -----------------------------------------------------------------
+    def _fused(self, lins, x):
+        """Several LutLinears sharing the input x [B, K] in one launch."""
+        outs = [torch.zeros((x.shape[0], l.N), dtype=torch.float16, device=x.device) for l in lins]
+        arr = (native.RowwiseProblem * len(lins))()
+        for i, (l, o) in enumerate(zip(lins, outs)):
+            arr[i] = native.RowwiseProblem(l.binaryWeight.data_ptr(), l.alpha.data_ptr(), x.data_ptr(),
+                                           o.data_ptr(), l.N, l.K, l.wbit, l.num_groups, x.shape[0])
+        rc = native.cabi().lutgemm_gemv_rowwise_f16_grouped(
+            len(lins), arr, ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+        if rc:
+            raise RuntimeError(native.cabi().lutgemm_strerror(rc).decode())
+        return outs
+
+    def _linears(self, lins, x):
+        if self.fuse and len(lins) > 1:
+            return self._fused(lins, x)
+        return [l(x) for l in lins]
+
+    def _rope(self, t, cos, sin):
+        half = t.shape[-1] // 2
+        rot = torch.cat([-t[..., half:], t[..., :half]], dim=-1)
+        return t * cos + rot * sin
+
+    # ---- one token ---------------------------------------------------------------------------
+    @torch.no_grad()
+    def step(self):
+        """Consumes self.ids [B] at position self.pos [1]; writes self.logits [B, V]."""
+        cfg, B = self.cfg, self.batch
+        hd, H, KV = cfg.head_dim, cfg.heads, cfg.kv_heads
+        x = self.embed[self.ids]                                    # [B, hidden]
+        cos = self.cos.index_select(0, self.pos).view(1, 1, hd)
+        sin = self.sin.index_select(0, self.pos).view(1, 1, hd)
+        # keys at positions > pos are masked out
+        mask = (self.positions <= self.pos).view(1, 1, 1, cfg.max_positions)
+        for li, blk in enumerate(self.blocks):
+            h = rms_norm(x, blk.input_norm, cfg.rms_eps).contiguous()
+            q, k, v = self._linears([blk.q_proj, blk.k_proj, blk.v_proj], h)
+            q = self._rope(q.view(B, H, hd), cos, sin)
+            k = self._rope(k.view(B, KV, hd), cos, sin)
+            self.k_cache[li].index_copy_(2, self.pos, k.unsqueeze(2))
+            self.v_cache[li].index_copy_(2, self.pos, v.view(B, KV, 1, hd))
+            kk, vv = self.k_cache[li], self.v_cache[li]
+            if KV != H:
+                kk = kk.repeat_interleave(H // KV, dim=1)
+                vv = vv.repeat_interleave(H // KV, dim=1)
+            att = F.scaled_dot_product_attention(q.unsqueeze(2), kk, vv, attn_mask=mask)   # [B, H, 1, hd]
+            (o,) = self._linears([blk.o_proj], att.reshape(B, H * hd).contiguous())
+            x = x + o
+            h = rms_norm(x, blk.post_norm, cfg.rms_eps).contiguous()
+            g, u = self._linears([blk.gate_proj, blk.up_proj], h)
+            (d,) = self._linears([blk.down_proj], (F.silu(g) * u).contiguous())
+            x = x + d
+        x = rms_norm(x, self.final_norm, cfg.rms_eps)
+        self.logits.copy_(x @ self.lm_head.t())
+
+    @torch.no_grad()
+    def capture(self):
+        """Capture step() in a HIP graph (after one eager run on the capture stream,
+        which also sizes the LUT-GEMM workspace of that stream)."""
+        self._stream = torch.cuda.Stream()
+        with torch.cuda.stream(self._stream):
+            self.step()
+        self._stream.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g, stream=self._stream):
+            self.step()
+        self._graph = g
+
+    @torch.no_grad()
+    def forward_token(self, ids: torch.Tensor, position: int):
+        self.ids.copy_(ids)
+        self.pos.fill_(position)
+        if self._graph is not None:
+            self._graph.replay()
+        else:
+            self.step()
+        return self.logits
+
+    def reset(self):
+        self.k_cache.zero_()
+        self.v_cache.zero_()
+
+    def linear_bytes_per_token(self):
+        """Algorithmic HBM bytes of the LUT-GEMM calls of one step (signs + alphas
+        + activations + outputs), for throughput accounting."""
+        lib = native.cabi()
+        total = 0
+        for blk in self.blocks:
+            for l in (blk.q_proj, blk.k_proj, blk.v_proj, blk.o_proj, blk.gate_proj, blk.up_proj, blk.down_proj):
+                total += lib.lutgemm_algorithmic_bytes(l.N, l.K, l.wbit, self.batch, l.num_groups * l.wbit * l.N, 2)
+        return total
+
+
+@torch.no_grad()
+def benchmark(model: LutDecoder, input_ids: torch.Tensor, generate: int = 128, warmup: int = 10):
+    """input_ids [B, T] prompt.  Every prompt token, then `generate` greedy tokens,
+    is one synchronised single-token step.  Returns a dict with the median seconds
+    per token over the generated tokens (and over the prompt tokens), tokens/s
+    (batch * 1/median) and the generated ids."""
+    B, T = input_ids.shape
+    assert B == model.batch and T + generate <= model.cfg.max_positions
+    dev = model.ids.device
+    input_ids = input_ids.to(dev)
+    for _ in range(warmup):
+        model.forward_token(input_ids[:, 0], 0)
+        torch.cuda.synchronize()
+    model.reset()
+    times_prompt, times_gen, out_ids = [], [], []
+    nxt = None
+    for i in range(T + generate):
+        ids = input_ids[:, i] if i < T else nxt
+        torch.cuda.synchronize()
+        tick = time.perf_counter()
+        logits = model.forward_token(ids, i)
+        torch.cuda.synchronize()
+        (times_prompt if i < T else times_gen).append(time.perf_counter() - tick)
+        nxt = logits.argmax(dim=-1)
+        if i >= T - 1:
+            out_ids.append(nxt.clone())
+    med = statistics.median(times_gen) if times_gen else float("nan")
+    return {
+        "batch": B, "prompt_tokens": T, "generated_tokens": generate,
+        "median_s_per_token": med,
+        "median_s_per_prompt_token": statistics.median(times_prompt),
+        "tokens_per_s": B / med if med == med else float("nan"),
+        "generated": torch.stack(out_ids[:-1], dim=1).cpu() if len(out_ids) > 1 else None,
+    }
