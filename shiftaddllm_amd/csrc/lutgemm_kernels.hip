@@ -63,6 +63,7 @@ constexpr int kWaveCols = 32;              // outputs a wave covers per step
 constexpr int kStepCols = kWaves * kWaveCols;  // outputs a workgroup covers per step
 constexpr int kEntryStride = 64;           // dwords between consecutive entries of a table
 constexpr int kLutDwords = 256 * kEntryStride;  // 64 KiB: two interleaved table buffers
+constexpr int kStageDwords = 2 * 2 * 4 * kTables;  // staged block alphas: [buffer][row group][bit][chunk]
 constexpr int kMaxKSplit = 32;             // bounded by the fixed-point accumulator layout
 constexpr int kMaxGroup = LUTGEMM_MAX_GROUP;  // problems per grouped launch
 
@@ -78,7 +79,16 @@ enum AlphaMode : int {
     kBlockShiftU16 = 2,
     kBlockApotI8 = 3,
     kUniformF16 = 4,  // alpha, q_bias fp16 [G][N]
+    // block formats when an N-tile spans at most two alpha row groups: the set's
+    // alphas are staged in LDS by the workgroup instead of loaded lane by lane
+    kBlockF16Staged = 5,
+    kBlockShiftU16Staged = 6,
+    kBlockApotI8Staged = 7,
 };
+
+constexpr bool is_block(int mode) { return mode == kBlockF16 || mode == kBlockShiftU16 || mode == kBlockApotI8; }
+constexpr bool is_staged(int mode) { return mode >= kBlockF16Staged; }
+constexpr int base_mode(int mode) { return is_staged(mode) ? mode - 4 : mode; }
 
 struct Problem {
     const uint32_t *W;
@@ -156,6 +166,7 @@ struct SetOperands {
     float a_blk[NSTEPS][NB][4]; // block: one multiplier per look-up step
     u32x2 a_uni[NSTEPS];        // uniform: alpha per output
     u32x2 q_uni[NSTEPS];        // uniform: q_bias per output
+    float a_stage;              // staged block modes: the one alpha this thread stages
 };
 
 // Per-lane address parts that do not change from set to set.
@@ -163,7 +174,9 @@ template <int NSTEPS>
 struct LaneCols {
     uint32_t col4[NSTEPS];  // byte offset of the lane's output quad inside a row of sign words
     uint32_t col2[NSTEPS];  // same, inside a row of fp16 alphas
-    int rgroup[NSTEPS];     // block modes: alpha row group of the quad
+    int rgroup[NSTEPS];     // block modes: alpha row group of the quad (staged: relative to the tile's first)
+    int rg0;                // staged block modes: first row group of the tile
+    int tid;
 };
 
 // Issue every global load of one table set for this lane.  Branch-free on
@@ -201,7 +214,7 @@ __device__ __forceinline__ void load_set(SetOperands<NB, NSTEPS, MODE> &r, const
             const uint32_t arow = (uint32_t)g * ((uint32_t)p.N * 2u);
             r.a_uni[s] = *(const u32x2 *)((const char *)p.alpha + (arow + lc.col2[s]));
             r.q_uni[s] = *(const u32x2 *)((const char *)p.qbias + (arow + lc.col2[s]));
-        } else {
+        } else if constexpr (is_block(MODE)) {
 #pragma unroll
             for (int b = 0; b < NB; ++b)
 #pragma unroll
@@ -210,6 +223,27 @@ __device__ __forceinline__ void load_set(SetOperands<NB, NSTEPS, MODE> &r, const
                     r.a_blk[s][b][j] =
                         load_block_alpha<MODE>(p.alpha, ((size_t)chunk * NB + b) * p.R + lc.rgroup[s]);
                 }
+        }
+    }
+    if constexpr (is_staged(MODE)) {
+        // thread t stages alpha(chunk c of the set, bit b, row group rg0 + g2)
+        const int t = lc.tid % (2 * NB * kTables);
+        const int c = t % kTables, b = (t / kTables) % NB, g2 = t / (NB * kTables);
+        const int chunk = min(set * kTables + c, p.K / 8 - 1);
+        const int rg = min(lc.rg0 + g2, p.R - 1);
+        r.a_stage = load_block_alpha<base_mode(MODE)>(p.alpha, ((size_t)chunk * NB + b) * p.R + rg);
+    }
+}
+
+// Staged block modes: publish this thread's alpha of a set into stage buffer `abuf`.
+template <int NB, int NSTEPS, int MODE>
+__device__ __forceinline__ void stage_alpha(const SetOperands<NB, NSTEPS, MODE> &ops, float *stage, int abuf,
+                                            int tid)
+{
+    if constexpr (is_staged(MODE)) {
+        if (tid < 2 * NB * kTables) {
+            const int c = tid % kTables, b = (tid / kTables) % NB, g2 = tid / (NB * kTables);
+            stage[((abuf * 2 + g2) * 4 + b) * kTables + c] = ops.a_stage;
         }
     }
 }
@@ -275,12 +309,14 @@ __device__ __forceinline__ void build_tables(const u32x4 &xraw, float *lut, int 
 template <int NB, int NSTEPS, int MODE>
 __device__ __forceinline__ void lookup_set(const SetOperands<NB, NSTEPS, MODE> &cur, const float *lut,
                                            float (&acc)[NSTEPS][4], uint32_t lane_off,
-                                           const uint32_t (&sel)[4])
+                                           const uint32_t (&sel)[4], const float *stage_lane,
+                                           const LaneCols<NSTEPS> &lc)
 {
     const char *lut_bytes = (const char *)lut;
     constexpr int kUnits = NSTEPS * NB;
     float val[2][16];
-    auto issue = [&](int u, float (&v)[16]) {
+    [[maybe_unused]] float aval[2][4];
+    auto issue = [&](int u, float (&v)[16], float (&av)[4]) {
         const int s = u / NB, b = u % NB;
         const uint32_t w4[4] = {cur.w[s][b].x, cur.w[s][b].y, cur.w[s][b].z, cur.w[s][b].w};
 #pragma unroll
@@ -288,8 +324,15 @@ __device__ __forceinline__ void lookup_set(const SetOperands<NB, NSTEPS, MODE> &
 #pragma unroll
             for (int j = 0; j < 4; ++j)
                 v[4 * i + j] = *(const float *)(lut_bytes + __builtin_amdgcn_perm(w4[i], lane_off, sel[j]));
+        if constexpr (is_staged(MODE)) {
+            // stage_lane points at [this set's buffer][group 0][bit 0][kw*4]; the four
+            // alphas of the lane's sign word, in look-up step order
+            const float *a4 = stage_lane + (lc.rgroup[s] * 4 + b) * kTables;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) av[j] = a4[(j + (lc.tid & 3)) & 3];
+        }
     };
-    auto retire = [&](int u, const float (&v)[16]) {
+    auto retire = [&](int u, const float (&v)[16], const float (&av)[4]) {
         const int s = u / NB, b = u % NB;
         [[maybe_unused]] const uint32_t ar[2] = {cur.a_row[s][b].x, cur.a_row[s][b].y};
         [[maybe_unused]] const uint32_t au[2] = {cur.a_uni[s].x, cur.a_uni[s].y};
@@ -302,13 +345,15 @@ __device__ __forceinline__ void lookup_set(const SetOperands<NB, NSTEPS, MODE> &
                 a = half_bits_to_float((au[i >> 1] >> (16 * (i & 1))) & 0xffffu) * (1.0f / (float)(2 << b));
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
-                if constexpr (MODE == kBlockF16 || MODE == kBlockShiftU16 || MODE == kBlockApotI8)
+                if constexpr (is_block(MODE))
                     a = cur.a_blk[s][b][j];
+                else if constexpr (is_staged(MODE))
+                    a = av[j];
                 acc[s][i] = fmaf(v[4 * i + j], a, acc[s][i]);
             }
         }
     };
-    issue(0, val[0]);
+    issue(0, val[0], aval[0]);
     if constexpr (MODE == kUniformF16) {
         // sum of the lane's 32 inputs = entry 255 of its four tables
         float sum_x = 0.0f;
@@ -325,8 +370,8 @@ __device__ __forceinline__ void lookup_set(const SetOperands<NB, NSTEPS, MODE> &
     }
 #pragma unroll
     for (int u = 0; u < kUnits; ++u) {
-        if (u + 1 < kUnits) issue(u + 1, val[(u + 1) & 1]);
-        retire(u, val[u & 1]);
+        if (u + 1 < kUnits) issue(u + 1, val[(u + 1) & 1], aval[(u + 1) & 1]);
+        retire(u, val[u & 1], aval[u & 1]);
     }
 }
 
@@ -383,9 +428,14 @@ __device__ __forceinline__ void gemv_tile(const Problem &p, int tile, int kslice
         const int n = min(n_lane + s * kStepCols, p.N - 4);
         lc.col4[s] = (uint32_t)n * 4u;
         lc.col2[s] = (uint32_t)n * 2u;
-        lc.rgroup[s] = (MODE == kBlockF16 || MODE == kBlockShiftU16 || MODE == kBlockApotI8)
-                           ? n / p.rows_per_group : 0;
+        lc.rgroup[s] = 0;
+        if constexpr (is_block(MODE)) lc.rgroup[s] = n / p.rows_per_group;
+        if constexpr (is_staged(MODE)) lc.rgroup[s] = n / p.rows_per_group - tile0 / p.rows_per_group;
     }
+    lc.rg0 = is_staged(MODE) ? tile0 / p.rows_per_group : 0;
+    lc.tid = tid;
+    float *stage = lut + kLutDwords;
+    int abuf = 0;
 
     // Two operand buffers used alternately: while set i is looked up, the loads of
     // set i+1 are in flight.  No register copies between them (a copy would have
@@ -405,13 +455,15 @@ __device__ __forceinline__ void gemv_tile(const Problem &p, int tile, int kslice
 
     int buf = 0;
     build_tables(load_x_chunk(p, xrow[0], set_begin, tb), lut, 0, tb, eb);
+    stage_alpha<NB, NSTEPS, MODE>(opA, stage, 0, tid);
     __syncthreads();
     // Steady state, per (set, row) item: fetch the activations of the next item,
     // look the current item up in table buffer f, build the next item's tables into
     // buffer f^1, one barrier.  The barrier both publishes buffer f^1 and retires
     // the readers of buffer f, which the item after next overwrites.
     constexpr uint32_t kFlip = 0x80808080u;  // +128 bytes = the other table buffer
-    auto rows_of_set = [&](const SetOperands<NB, NSTEPS, MODE> &ops, int set, auto has_next_set) {
+    auto rows_of_set = [&](const SetOperands<NB, NSTEPS, MODE> &ops, const SetOperands<NB, NSTEPS, MODE> &nxt,
+                           int set, auto has_next_set) {
 #pragma unroll
         for (int r = 0; r < MROWS; ++r) {
             const bool more = (r + 1 < MROWS) || decltype(has_next_set)::value;
@@ -422,29 +474,34 @@ __device__ __forceinline__ void gemv_tile(const Problem &p, int tile, int kslice
             // opaque to the optimiser: otherwise the 48 look-up addresses of a set are
             // kept in registers across all rows instead of being recomputed (1 op each)
             asm volatile("" : "+v"(lane_off));
-            lookup_set<NB, NSTEPS, MODE>(ops, lut, acc[r], lane_off, sel);
+            lookup_set<NB, NSTEPS, MODE>(ops, lut, acc[r], lane_off, sel,
+                                         stage + abuf * (2 * 4 * kTables) + kw * 4, lc);
             if (more) {
                 buf ^= 1;
                 lane_off ^= kFlip;
                 build_tables(xn, lut, buf, tb, eb);
+                if (r + 1 == MROWS) {  // moving on to the next set: its alphas go to the other stage buffer
+                    abuf ^= 1;
+                    stage_alpha<NB, NSTEPS, MODE>(nxt, stage, abuf, tid);
+                }
                 __syncthreads();
             }
         }
     };
     for (int set = set_begin;;) {
         if (set + 1 >= set_end) {
-            rows_of_set(opA, set, std::false_type{});
+            rows_of_set(opA, opA, set, std::false_type{});
             break;
         }
         load_set<NB, NSTEPS, MODE>(opB, p, set + 1, kw, q, lc);
-        rows_of_set(opA, set, std::true_type{});
+        rows_of_set(opA, opB, set, std::true_type{});
         ++set;
         if (set + 1 >= set_end) {
-            rows_of_set(opB, set, std::false_type{});
+            rows_of_set(opB, opB, set, std::false_type{});
             break;
         }
         load_set<NB, NSTEPS, MODE>(opA, p, set + 1, kw, q, lc);
-        rows_of_set(opB, set, std::true_type{});
+        rows_of_set(opB, opA, set, std::true_type{});
         ++set;
     }
 
@@ -529,7 +586,7 @@ __device__ __forceinline__ void gemv_tile(const Problem &p, int tile, int kslice
 template <int NB, int NSTEPS, int MODE, int MROWS>
 __global__ void __launch_bounds__(kThreads) lut_gemv_kernel(const Problem p)
 {
-    __shared__ __attribute__((aligned(16))) float lut[kLutDwords];
+    __shared__ __attribute__((aligned(16))) float lut[kLutDwords + kStageDwords];
     int tile, kslice, mchunk;
     decode_block(p, (int)blockIdx.x, tile, kslice, mchunk);
     gemv_tile<NB, NSTEPS, MODE, MROWS>(p, tile, kslice, mchunk, lut);
@@ -540,7 +597,7 @@ __global__ void __launch_bounds__(kThreads) lut_gemv_kernel(const Problem p)
 template <int NSTEPS>
 __global__ void __launch_bounds__(kThreads) lut_gemv_group_kernel(const Group g)
 {
-    __shared__ __attribute__((aligned(16))) float lut[kLutDwords];
+    __shared__ __attribute__((aligned(16))) float lut[kLutDwords + kStageDwords];
     const int b = blockIdx.x;
     int pi = 0;
 #pragma unroll
@@ -754,7 +811,11 @@ int run(int mode, const uint32_t *bW, const void *alpha, const void *qbias, cons
         rc = get_workspace(stream, (size_t)M * N, &p.accum);
         if (rc != LUTGEMM_OK) return rc;
     }
+    if (is_block(mode) && p.rows_per_group >= kStepCols * nsteps) mode += 4;  // tile spans <= 2 row groups
     switch (mode) {
+    case kBlockF16Staged: return launch_mode<kBlockF16Staged>(p, nsteps, mrows, stream);
+    case kBlockShiftU16Staged: return launch_mode<kBlockShiftU16Staged>(p, nsteps, mrows, stream);
+    case kBlockApotI8Staged: return launch_mode<kBlockApotI8Staged>(p, nsteps, mrows, stream);
     case kRowF16: return launch_mode<kRowF16>(p, nsteps, mrows, stream);
     case kBlockF16: return launch_mode<kBlockF16>(p, nsteps, mrows, stream);
     case kBlockShiftU16: return launch_mode<kBlockShiftU16>(p, nsteps, mrows, stream);

@@ -199,7 +199,9 @@ def test_config3_non_square_shapes(gpu_device, N, K):
 
 
 @pytest.mark.parametrize("N,K,nb,R,M", [(32, 32, 1, 1, 1), (64, 96, 3, 4, 2), (640, 288, 2, 8, 1),
-                                         (256, 512, 4, 64, 3), (1024, 1024, 3, 8, 1)])
+                                         (256, 512, 4, 64, 3), (1024, 1024, 3, 8, 1),
+                                         (2560, 544, 3, 4, 3),     # tiles straddle row groups, several rows
+                                         (2048, 256, 4, 2, 5)])
 def test_block_f16_ragged(gpu_device, N, K, nb, R, M):
     p = workload.make_block_problem(N, K, nb=nb, R=R, M=M, seed=N + R, quantize=False)
     want, _ = orc.gemv_block_c(p.bW.numpy(), p.alpha.numpy(), p.x.numpy(), R, kind=orc.ALPHA_F16)
