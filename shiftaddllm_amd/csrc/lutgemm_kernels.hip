@@ -614,6 +614,222 @@ __global__ void __launch_bounds__(kThreads) lut_gemv_group_kernel(const Group g)
     }
 }
 
+// ---------------------------------------------------------------------------
+// Small-batch path (row-wise alpha, several activation rows): matrix cores.
+//
+// Table look-ups cost one LDS read and two VALU operations per sign byte PER
+// ROW, so beyond a couple of rows the look-up kernel is VALU/LDS bound
+// (measured: ~21 us per extra row on a 132 MB matrix whose stream takes 18 us).
+// Here the sign bits are expanded to +-1.0 fp16 in registers (one VALU
+// operation per two signs) and multiplied with 16 activation rows at a time by
+// v_mfma_f32_16x16x32_f16, fp32 accumulation; alpha scales each (group, bit
+// plane) partial product with one fma per output.
+//
+// Work split: workgroup = 4 waves x 64 outputs; a K-step is 128 inputs (4 sign
+// words = one alpha group of 128).  Lane l (li = l&15, kb = l>>4) loads the four
+// sign words of outputs n = base + 4*li .. +3 for word kb of the step (256-byte
+// runs per row).  MFMA instance (e, beta) takes from every lane 8 signs of its
+// word e: bits 4*beta+i and 16+4*beta+i, i < 4 -- two bits 16 apart land in the
+// sign positions of a packed fp16 pair with ONE shift and ONE and-or.  So the
+// instance's A rows are outputs base + 4*i + e and its K block kb is word kb;
+// the activations are staged in LDS in exactly that K order.
+// ---------------------------------------------------------------------------
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+constexpr int kMfmaThreads = 256;
+constexpr int kMfmaWaves = kMfmaThreads / 64;
+constexpr int kMfmaWaveCols = 64;
+constexpr int kMfmaTileCols = kMfmaWaves * kMfmaWaveCols;  // 256 outputs per workgroup
+constexpr int kMfmaStepK = 128;
+constexpr int kXRowBytes = 256 + 16;  // one activation row of a K-step, padded against bank conflicts
+
+template <int NB>
+struct MfmaOperands {
+    u32x4 w[NB];      // sign words of 4 outputs
+    u32x2 a[NB][4];   // 16 fp16 alphas: outputs base + 16*kb .. +15
+};
+
+template <int NB>
+__device__ __forceinline__ void mfma_load_step(MfmaOperands<NB> &r, const Problem &p, int step, int kb,
+                                               uint32_t wcol4, uint32_t acol2)
+{
+    const uint32_t row_bytes = (uint32_t)p.N * 4u;
+    const char *wbase = (const char *)p.W + (size_t)step * 4 * NB * row_bytes;
+    const uint32_t wrow = (uint32_t)kb * (NB * row_bytes);
+    const int g = (step * 4) / p.group_words;
+    const uint32_t arow = (uint32_t)g * (NB * (uint32_t)p.N * 2u);
+#pragma unroll
+    for (int b = 0; b < NB; ++b) {
+        r.w[b] = __builtin_nontemporal_load((const u32x4 *)(wbase + (size_t)b * row_bytes + (wrow + wcol4)));
+        const char *asrc = (const char *)p.alpha + (size_t)b * p.N * 2u + (arow + acol2);
+#pragma unroll
+        for (int v = 0; v < 4; ++v) r.a[b][v] = *(const u32x2 *)(asrc + 8 * v);
+    }
+}
+
+// 8 signs of `wn` (the complemented sign word) -> 8 fp16 +-1.0: pair i holds
+// bit 4*beta+i (low half) and bit 16+4*beta+i (high half).
+__device__ __forceinline__ f16x8 expand_signs(uint32_t wn, int beta)
+{
+    u32x4 r;
+    r.x = ((wn << (15 - (4 * beta + 0))) & 0x80008000u) | 0x3c003c00u;
+    r.y = ((wn << (15 - (4 * beta + 1))) & 0x80008000u) | 0x3c003c00u;
+    r.z = ((wn << (15 - (4 * beta + 2))) & 0x80008000u) | 0x3c003c00u;
+    r.w = ((wn << (15 - (4 * beta + 3))) & 0x80008000u) | 0x3c003c00u;
+    return __builtin_bit_cast(f16x8, r);
+}
+
+template <int NB, int MT>
+__global__ void __launch_bounds__(kMfmaThreads) lut_gemm_mfma_kernel(const Problem p)
+{
+    __shared__ __attribute__((aligned(16))) char xs[2][16 * MT * kXRowBytes];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int li = lane & 15;
+    const int kb = lane >> 4;
+    int tile, kslice, mchunk;
+    decode_block(p, (int)blockIdx.x, tile, kslice, mchunk);
+    const int m0 = mchunk * 16 * MT;
+    const int n_base = tile * kMfmaTileCols + wave * kMfmaWaveCols;
+
+    const uint32_t wcol4 = (uint32_t)min(n_base + 4 * li, p.N - 4) * 4u;
+    const uint32_t acol2 = (uint32_t)min(n_base + 16 * kb, p.N - 16) * 2u;
+
+    const int step_begin = kslice * p.sets_per_split;
+    const int step_end = min(step_begin + p.sets_per_split, p.nsets);
+
+    // activation staging: target t = (row rr, word w, instance beta) gets 8 halves in MFMA K order
+    u32x2 xlo[MT], xhi[MT];
+    auto x_fetch = [&](int step) {
+#pragma unroll
+        for (int u = 0; u < MT; ++u) {
+            const int t = tid + kMfmaThreads * u;
+            const int rr = t >> 4, w = (t >> 2) & 3, beta = t & 3;
+            const __half *src = p.x + (size_t)min(m0 + rr, p.M - 1) * p.K + step * kMfmaStepK + 32 * w + 4 * beta;
+            xlo[u] = *(const u32x2 *)src;
+            xhi[u] = *(const u32x2 *)(src + 16);
+        }
+    };
+    auto x_publish = [&](int buf) {
+#pragma unroll
+        for (int u = 0; u < MT; ++u) {
+            const int t = tid + kMfmaThreads * u;
+            const int rr = t >> 4, w = (t >> 2) & 3, beta = t & 3;
+            u32x4 v;
+            v.x = __builtin_amdgcn_perm(xhi[u].x, xlo[u].x, 0x05040100u);
+            v.y = __builtin_amdgcn_perm(xhi[u].x, xlo[u].x, 0x07060302u);
+            v.z = __builtin_amdgcn_perm(xhi[u].y, xlo[u].y, 0x05040100u);
+            v.w = __builtin_amdgcn_perm(xhi[u].y, xlo[u].y, 0x07060302u);
+            *(u32x4 *)(xs[buf] + rr * kXRowBytes + w * 64 + beta * 16) = v;
+        }
+    };
+
+    f32x4 acc[4][MT];
+#pragma unroll
+    for (int e = 0; e < 4; ++e)
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) acc[e][mt] = (f32x4){0.0f, 0.0f, 0.0f, 0.0f};
+
+    auto compute = [&](const MfmaOperands<NB> &ops, int buf) {
+        f16x8 bx[MT][4];
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+            for (int beta = 0; beta < 4; ++beta)
+                bx[mt][beta] = *(const f16x8 *)(xs[buf] + (16 * mt + li) * kXRowBytes + kb * 64 + beta * 16);
+#pragma unroll
+        for (int b = 0; b < NB; ++b) {
+            const uint32_t w4[4] = {~ops.w[b].x, ~ops.w[b].y, ~ops.w[b].z, ~ops.w[b].w};
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                f32x4 d[MT];
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt) d[mt] = (f32x4){0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+                for (int beta = 0; beta < 4; ++beta) {
+                    const f16x8 a = expand_signs(w4[e], beta);
+#pragma unroll
+                    for (int mt = 0; mt < MT; ++mt)
+                        d[mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, bx[mt][beta], d[mt], 0, 0, 0);
+                }
+                // D row 4*kb + r is output base + 16*kb + 4*r + e: alpha number 4*r + e of the lane's 16
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const int idx = 4 * r + e;
+                    const uint32_t raw = (idx & 2) ? ops.a[b][idx >> 2].y : ops.a[b][idx >> 2].x;
+                    const float al = half_bits_to_float((raw >> (16 * (idx & 1))) & 0xffffu);
+#pragma unroll
+                    for (int mt = 0; mt < MT; ++mt) acc[e][mt][r] = fmaf(d[mt][r], al, acc[e][mt][r]);
+                }
+            }
+        }
+    };
+
+    MfmaOperands<NB> opA, opB;
+    mfma_load_step<NB>(opA, p, step_begin, kb, wcol4, acol2);
+    x_fetch(step_begin);
+    x_publish(0);
+    __syncthreads();
+    for (int step = step_begin;;) {
+        if (step + 1 >= step_end) {
+            compute(opA, 0);
+            break;
+        }
+        mfma_load_step<NB>(opB, p, step + 1, kb, wcol4, acol2);
+        x_fetch(step + 1);
+        compute(opA, 0);
+        x_publish(1);
+        __syncthreads();
+        ++step;
+        if (step + 1 >= step_end) {
+            compute(opB, 1);
+            break;
+        }
+        mfma_load_step<NB>(opA, p, step + 1, kb, wcol4, acol2);
+        x_fetch(step + 1);
+        compute(opB, 1);
+        x_publish(0);
+        __syncthreads();
+        ++step;
+    }
+
+    // ---- write: lane holds, for rows m = m0 + 16*mt + li, outputs n_base + 16*kb + 4*r + e ----
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+        const int m = m0 + 16 * mt + li;
+        if (m >= p.M) continue;
+        __half *out = p.out + (size_t)m * p.N;
+        unsigned long long *accum = p.accum + (size_t)m * p.N;
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const int n = n_base + 16 * kb + 4 * r + e;
+                if (n >= p.N) continue;
+                float v = acc[e][mt][r];
+                if (p.ksplit == 1) {
+                    out[n] = __float2half_rn(__half2float(out[n]) + v);
+                    continue;
+                }
+                v = (v == v) ? v : 65536.0f;
+                v = fminf(fmaxf(v, -65536.0f), 65536.0f);
+                const long long fx = __double2ll_rn((double)v * 4294967296.0);
+                const unsigned long long contrib = (unsigned long long)(fx + kBias) + kCountOne;
+                const unsigned long long old =
+                    __hip_atomic_fetch_add(accum + n, contrib, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                if ((int)(old >> 56) != p.ksplit - 1) continue;
+                const long long total = (long long)((old + contrib) & kSumMask) - (long long)p.ksplit * kBias;
+                const float y = (float)((double)total * (1.0 / 4294967296.0));
+                out[n] = __float2half_rn(__half2float(out[n]) + y);
+                __hip_atomic_store(accum + n, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+    }
+}
+
+
 __global__ void __launch_bounds__(256) copy_kernel(u32x4 *dst, const u32x4 *src, size_t n16)
 {
     size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -797,6 +1013,59 @@ int fill_problem(Problem &p, int mode, const uint32_t *bW, const void *alpha, co
     return LUTGEMM_OK;
 }
 
+int mfma_min_rows()
+{
+    static const int v = env_int("LUTGEMM_MFMA_MIN_M", 3);
+    return v;
+}
+
+// The matrix-core path needs whole 128-input steps inside one alpha group and
+// 16-output alpha runs.
+bool mfma_eligible(const Problem &p, int mode)
+{
+    return mode == kRowF16 && p.M >= mfma_min_rows() && p.K % kMfmaStepK == 0 && p.group_words % 4 == 0 &&
+           p.N % 16 == 0 && p.N >= 16;
+}
+
+template <int NB>
+int launch_mfma_nb(const Problem &p, int mt, hipStream_t stream)
+{
+    dim3 grid((unsigned)p.n_blocks), block(kMfmaThreads);
+    if (mt == 2)
+        hipLaunchKernelGGL((lut_gemm_mfma_kernel<NB, 2>), grid, block, 0, stream, p);
+    else
+        hipLaunchKernelGGL((lut_gemm_mfma_kernel<NB, 1>), grid, block, 0, stream, p);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return hip_fail(e);
+    return LUTGEMM_OK;
+}
+
+int run_mfma(Problem &p, hipStream_t stream)
+{
+    const int mt = p.M > 16 ? 2 : 1;
+    p.n_tiles = (p.N + kMfmaTileCols - 1) / kMfmaTileCols;
+    p.mchunks = (p.M + 16 * mt - 1) / (16 * mt);
+    p.nsets = p.K / kMfmaStepK;  // K-steps
+    long want = (long)target_blocks() * 2 / ((long)p.n_tiles * p.mchunks);
+    if (want < 1) want = 1;
+    if (want > p.nsets) want = p.nsets;
+    if (want > kMaxKSplit) want = kMaxKSplit;
+    p.sets_per_split = (p.nsets + (int)want - 1) / (int)want;
+    p.ksplit = (p.nsets + p.sets_per_split - 1) / p.sets_per_split;
+    p.n_blocks = p.n_tiles * p.ksplit * p.mchunks;
+    if (p.ksplit > 1) {
+        int rc = get_workspace(stream, (size_t)p.M * p.N, &p.accum);
+        if (rc != LUTGEMM_OK) return rc;
+    }
+    switch (p.nb) {
+    case 1: return launch_mfma_nb<1>(p, mt, stream);
+    case 2: return launch_mfma_nb<2>(p, mt, stream);
+    case 3: return launch_mfma_nb<3>(p, mt, stream);
+    case 4: return launch_mfma_nb<4>(p, mt, stream);
+    default: return LUTGEMM_EINVAL;
+    }
+}
+
 int run(int mode, const uint32_t *bW, const void *alpha, const void *qbias, const void *x,
         void *out, int N, int K, int nb, int num_groups, int M, void *stream_v)
 {
@@ -804,6 +1073,7 @@ int run(int mode, const uint32_t *bW, const void *alpha, const void *qbias, cons
     int rc = fill_problem(p, mode, bW, alpha, qbias, x, out, N, K, nb, num_groups, M);
     if (rc != LUTGEMM_OK) return rc;
     hipStream_t stream = (hipStream_t)stream_v;
+    if (mfma_eligible(p, mode)) return run_mfma(p, stream);
     const int mrows = pick_mrows(M);
     const int nsteps = mrows > 1 ? 1 : pick_nsteps(N);
     plan_problem(p, nsteps, mrows, target_blocks());

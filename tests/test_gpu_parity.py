@@ -177,6 +177,34 @@ def test_config5_small_batches(gpu_device, M):
     _assert_close(run_rowwise(gpu_device, p.bW, p.alpha, p.x, p.num_groups), want)
 
 
+@pytest.mark.parametrize("N,K,nb,gs,M", [
+    (16, 128, 1, 128, 3),        # smallest problem the matrix-core path takes
+    (80, 256, 2, 128, 5),        # N not a multiple of the wave tile, odd row count
+    (256, 1024, 3, 128, 16),
+    (1024, 4096, 4, 128, 17),    # second row chunk almost empty
+    (272, 384, 3, 128, 33),      # three row chunks, ragged N
+    (4096, 4096, 3, 256, 8),     # group of 256 inputs (two K-steps per alpha)
+    (11008, 4096, 2, 4096, 32),  # one group along K
+])
+def test_small_batch_matrix_core_path(gpu_device, N, K, nb, gs, M):
+    p = workload.make_rowwise_problem(N, K, nb=nb, group_size=gs, M=M, seed=N + M, quantize=False)
+    bias = torch.randn((M, N), generator=torch.Generator().manual_seed(M)).half()
+    want, _ = orc.gemv_rowwise_c(p.bW.numpy(), p.alpha.numpy(), p.x.numpy(), p.num_groups, out=bias.numpy())
+    got = run_rowwise(gpu_device, p.bW, p.alpha, p.x, p.num_groups, out=bias)
+    _assert_close(got, want, (N, K, nb, gs, M))
+    assert torch.equal(got, run_rowwise(gpu_device, p.bW, p.alpha, p.x, p.num_groups, out=bias))
+
+
+def test_batch_rows_agree_with_single_row_calls(gpu_device):
+    # every row of a batched call equals the batch-1 call on that row (different kernels)
+    p = workload.make_rowwise_problem(2048, 2048, nb=3, group_size=128, M=8, seed=77, quantize=False)
+    batched = run_rowwise(gpu_device, p.bW, p.alpha, p.x, p.num_groups).float().cpu()
+    for m in (0, 3, 7):
+        single = run_rowwise(gpu_device, p.bW, p.alpha, p.x[m:m + 1], p.num_groups).float().cpu()
+        rel, _ = orc.error_metrics(batched[m:m + 1].numpy(), single.numpy())
+        assert rel <= 2e-4, (m, rel)
+
+
 # ---- block alpha (config 3 and the LutLinear default format) -----------------
 
 def test_config3_llama13b_block_real_bcq(gpu_device):
