@@ -50,7 +50,7 @@ def parse_args():
     ap.add_argument("--plain-only", action="store_true",
                     help="only the 224-launch step (no fused sequences, no per-shape table): for profiler runs")
     ap.add_argument("--profile-shape", type=str, default="",
-                    help="N,K[,nb[,iters]]: only launch this shape repeatedly (for rocprofv3 runs) and exit")
+                    help="N,K[,nb[,iters[,M]]]: only launch this shape repeatedly (for rocprofv3 runs) and exit")
     ap.add_argument("--profile-copy", type=int, default=0,
                     help="bytes: only run the calibration copy kernel a few times (for rocprofv3 --pmc) and exit")
     return ap.parse_args()
@@ -59,9 +59,9 @@ def parse_args():
 class Gemv:
     """Device operands of one row-wise-alpha LUT-GEMV."""
 
-    def __init__(self, torch, dev, N, K, nb, seed, x=None):
+    def __init__(self, torch, dev, N, K, nb, seed, x=None, M=1):
         g = torch.Generator(device=dev).manual_seed(seed)
-        self.N, self.K, self.nb = N, K, nb
+        self.N, self.K, self.nb, self.M = N, K, nb, M
         self.groups = K // GROUP
         self.bW = torch.randint(-2 ** 31, 2 ** 31 - 1, (K // 32, nb, N), generator=g, device=dev,
                                 dtype=torch.int32)
@@ -69,13 +69,13 @@ class Gemv:
         e = torch.randint(-9, -5, (self.groups, 1, N), generator=g, device=dev).float()
         e = e - torch.arange(nb, device=dev).float().view(1, nb, 1)
         self.alpha = torch.exp2(e).to(torch.float16).contiguous()
-        self.x = x if x is not None else torch.randn((1, K), generator=g, device=dev).half()
-        self.out = torch.zeros((1, N), dtype=torch.float16, device=dev)
+        self.x = x if x is not None else torch.randn((M, K), generator=g, device=dev).half()
+        self.out = torch.zeros((M, N), dtype=torch.float16, device=dev)
         self.bytes = None
 
     def args(self):
         p = lambda t: ctypes.c_void_p(t.data_ptr())
-        return (p(self.bW), p(self.alpha), p(self.x), p(self.out), self.N, self.K, self.nb, self.groups, 1)
+        return (p(self.bW), p(self.alpha), p(self.x), p(self.out), self.N, self.K, self.nb, self.groups, self.M)
 
 
 def main():
@@ -122,12 +122,13 @@ def main():
         N, K = parts[0], parts[1]
         nb = parts[2] if len(parts) > 2 else NB
         iters = parts[3] if len(parts) > 3 else 8
-        pool = [Gemv(torch, dev, N, K, nb, 100 + i) for i in range(iters)]
+        rows = parts[4] if len(parts) > 4 else 1
+        pool = [Gemv(torch, dev, N, K, nb, 100 + i, M=rows) for i in range(iters)]
         with torch.cuda.stream(stream):
             for g in pool:      # each launch touches weights never read before
                 run(g, sp)
         stream.synchronize()
-        print(json.dumps({"shape": [N, K, nb], "launches": iters, "algorithmic_bytes_per_launch": alg_bytes(pool[0])}))
+        print(json.dumps({"shape": [N, K, nb], "rows": rows, "launches": iters, "algorithmic_bytes_per_launch": alg_bytes(pool[0])}))
         return
 
     # ---- weight pool: `layers` decoder blocks x 7 linears -----------------

@@ -625,22 +625,24 @@ __global__ void __launch_bounds__(kThreads) lut_gemv_group_kernel(const Group g)
 // v_mfma_f32_16x16x32_f16, fp32 accumulation; alpha scales each (group, bit
 // plane) partial product with one fma per output.
 //
-// Work split: workgroup = 4 waves x 64 outputs; a K-step is 128 inputs (4 sign
-// words = one alpha group of 128).  Lane l (li = l&15, kb = l>>4) loads the four
-// sign words of outputs n = base + 4*li .. +3 for word kb of the step (256-byte
-// runs per row).  MFMA instance (e, beta) takes from every lane 8 signs of its
-// word e: bits 4*beta+i and 16+4*beta+i, i < 4 -- two bits 16 apart land in the
-// sign positions of a packed fp16 pair with ONE shift and ONE and-or.  So the
-// instance's A rows are outputs base + 4*i + e and its K block kb is word kb;
-// the activations are staged in LDS in exactly that K order.
+// Work split: a workgroup of 8 waves owns 64 outputs; its waves take different
+// K-steps (128 inputs = 4 sign words = one alpha group of 128) and their
+// accumulators meet in LDS at the end, so that the number of cross-workgroup
+// atomics does not grow with the K parallelism.  Lane l (li = l&15, kb = l>>4)
+// loads the four sign words of outputs n = base + 4*li .. +3 for word kb of its
+// step (256-byte runs per row).  MFMA instance (e, beta) takes from every lane 8
+// signs of its word e: bits 4*beta+i and 16+4*beta+i, i < 4 -- two bits 16 apart
+// land in the sign positions of a packed fp16 pair with ONE shift and ONE
+// and-or.  So the instance's A rows are outputs base + 4*i + e and its K block
+// kb is word kb; the activations of a round (8 steps) are staged in LDS in
+// exactly that K order.
 // ---------------------------------------------------------------------------
 typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 
-constexpr int kMfmaThreads = 256;
+constexpr int kMfmaThreads = 512;
 constexpr int kMfmaWaves = kMfmaThreads / 64;
-constexpr int kMfmaWaveCols = 64;
-constexpr int kMfmaTileCols = kMfmaWaves * kMfmaWaveCols;  // 256 outputs per workgroup
+constexpr int kMfmaTileCols = 64;     // outputs per workgroup
 constexpr int kMfmaStepK = 128;
 constexpr int kXRowBytes = 256 + 16;  // one activation row of a K-step, padded against bank conflicts
 
@@ -668,22 +670,27 @@ __device__ __forceinline__ void mfma_load_step(MfmaOperands<NB> &r, const Proble
     }
 }
 
-// 8 signs of `wn` (the complemented sign word) -> 8 fp16 +-1.0: pair i holds
+// 8 signs of sign word `w` -> 8 fp16 +-1.0 (bit set = +1.0): pair i holds
 // bit 4*beta+i (low half) and bit 16+4*beta+i (high half).
-__device__ __forceinline__ f16x8 expand_signs(uint32_t wn, int beta)
+__device__ __forceinline__ f16x8 expand_signs(uint32_t w, int beta)
 {
+    // (~shifted & 0x80008000) | 0x3c003c00 as ONE three-input bit operation
+    // (truth table 0xae = (~a & b) | c); the compiler otherwise emits not + and + or.
+    const uint32_t sign = 0x80008000u, one = 0x3c003c00u;
     u32x4 r;
-    r.x = ((wn << (15 - (4 * beta + 0))) & 0x80008000u) | 0x3c003c00u;
-    r.y = ((wn << (15 - (4 * beta + 1))) & 0x80008000u) | 0x3c003c00u;
-    r.z = ((wn << (15 - (4 * beta + 2))) & 0x80008000u) | 0x3c003c00u;
-    r.w = ((wn << (15 - (4 * beta + 3))) & 0x80008000u) | 0x3c003c00u;
+    r.x = __builtin_amdgcn_bitop3_b32(w << (15 - (4 * beta + 0)), sign, one, 0xae);
+    r.y = __builtin_amdgcn_bitop3_b32(w << (15 - (4 * beta + 1)), sign, one, 0xae);
+    r.z = __builtin_amdgcn_bitop3_b32(w << (15 - (4 * beta + 2)), sign, one, 0xae);
+    r.w = __builtin_amdgcn_bitop3_b32(w << (15 - (4 * beta + 3)), sign, one, 0xae);
     return __builtin_bit_cast(f16x8, r);
 }
 
 template <int NB, int MT>
 __global__ void __launch_bounds__(kMfmaThreads) lut_gemm_mfma_kernel(const Problem p)
 {
-    __shared__ __attribute__((aligned(16))) char xs[2][16 * MT * kXRowBytes];
+    // activations of one round: [wave's step][row][word][instance][8 halves]; reused for the final reduction
+    constexpr int kWaveXBytes = 16 * MT * kXRowBytes;
+    __shared__ __attribute__((aligned(16))) char xs[kMfmaWaves * kWaveXBytes];
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -693,7 +700,7 @@ __global__ void __launch_bounds__(kMfmaThreads) lut_gemm_mfma_kernel(const Probl
     int tile, kslice, mchunk;
     decode_block(p, (int)blockIdx.x, tile, kslice, mchunk);
     const int m0 = mchunk * 16 * MT;
-    const int n_base = tile * kMfmaTileCols + wave * kMfmaWaveCols;
+    const int n_base = tile * kMfmaTileCols;
 
     const uint32_t wcol4 = (uint32_t)min(n_base + 4 * li, p.N - 4) * 4u;
     const uint32_t acol2 = (uint32_t)min(n_base + 16 * kb, p.N - 16) * 2u;
@@ -701,29 +708,23 @@ __global__ void __launch_bounds__(kMfmaThreads) lut_gemm_mfma_kernel(const Probl
     const int step_begin = kslice * p.sets_per_split;
     const int step_end = min(step_begin + p.sets_per_split, p.nsets);
 
-    // activation staging: target t = (row rr, word w, instance beta) gets 8 halves in MFMA K order
-    u32x2 xlo[MT], xhi[MT];
-    auto x_fetch = [&](int step) {
+    // Stage the activations of the round starting at step r0: target t = (step s of
+    // the round, row rr, word w, instance beta) gets 8 halves in MFMA K order.
+    auto stage_round = [&](int r0) {
 #pragma unroll
-        for (int u = 0; u < MT; ++u) {
+        for (int u = 0; u < 4 * MT; ++u) {
             const int t = tid + kMfmaThreads * u;
-            const int rr = t >> 4, w = (t >> 2) & 3, beta = t & 3;
+            const int beta = t & 3, w = (t >> 2) & 3, rr = (t >> 4) % (16 * MT), sidx = t / (256 * MT);
+            const int step = min(r0 + sidx, p.nsets - 1);
             const __half *src = p.x + (size_t)min(m0 + rr, p.M - 1) * p.K + step * kMfmaStepK + 32 * w + 4 * beta;
-            xlo[u] = *(const u32x2 *)src;
-            xhi[u] = *(const u32x2 *)(src + 16);
-        }
-    };
-    auto x_publish = [&](int buf) {
-#pragma unroll
-        for (int u = 0; u < MT; ++u) {
-            const int t = tid + kMfmaThreads * u;
-            const int rr = t >> 4, w = (t >> 2) & 3, beta = t & 3;
+            const u32x2 lo = *(const u32x2 *)src;
+            const u32x2 hi = *(const u32x2 *)(src + 16);
             u32x4 v;
-            v.x = __builtin_amdgcn_perm(xhi[u].x, xlo[u].x, 0x05040100u);
-            v.y = __builtin_amdgcn_perm(xhi[u].x, xlo[u].x, 0x07060302u);
-            v.z = __builtin_amdgcn_perm(xhi[u].y, xlo[u].y, 0x05040100u);
-            v.w = __builtin_amdgcn_perm(xhi[u].y, xlo[u].y, 0x07060302u);
-            *(u32x4 *)(xs[buf] + rr * kXRowBytes + w * 64 + beta * 16) = v;
+            v.x = __builtin_amdgcn_perm(hi.x, lo.x, 0x05040100u);
+            v.y = __builtin_amdgcn_perm(hi.x, lo.x, 0x07060302u);
+            v.z = __builtin_amdgcn_perm(hi.y, lo.y, 0x05040100u);
+            v.w = __builtin_amdgcn_perm(hi.y, lo.y, 0x07060302u);
+            *(u32x4 *)(xs + sidx * kWaveXBytes + rr * kXRowBytes + w * 64 + beta * 16) = v;
         }
     };
 
@@ -733,16 +734,17 @@ __global__ void __launch_bounds__(kMfmaThreads) lut_gemm_mfma_kernel(const Probl
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) acc[e][mt] = (f32x4){0.0f, 0.0f, 0.0f, 0.0f};
 
-    auto compute = [&](const MfmaOperands<NB> &ops, int buf) {
+    auto compute = [&](const MfmaOperands<NB> &ops) {
+        const char *xw = xs + wave * kWaveXBytes;
         f16x8 bx[MT][4];
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
             for (int beta = 0; beta < 4; ++beta)
-                bx[mt][beta] = *(const f16x8 *)(xs[buf] + (16 * mt + li) * kXRowBytes + kb * 64 + beta * 16);
+                bx[mt][beta] = *(const f16x8 *)(xw + (16 * mt + li) * kXRowBytes + kb * 64 + beta * 16);
 #pragma unroll
         for (int b = 0; b < NB; ++b) {
-            const uint32_t w4[4] = {~ops.w[b].x, ~ops.w[b].y, ~ops.w[b].z, ~ops.w[b].w};
+            const uint32_t w4[4] = {ops.w[b].x, ops.w[b].y, ops.w[b].z, ops.w[b].w};
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
                 f32x4 d[MT];
@@ -768,67 +770,58 @@ __global__ void __launch_bounds__(kMfmaThreads) lut_gemm_mfma_kernel(const Probl
         }
     };
 
-    MfmaOperands<NB> opA, opB;
-    mfma_load_step<NB>(opA, p, step_begin, kb, wcol4, acol2);
-    x_fetch(step_begin);
-    x_publish(0);
-    __syncthreads();
-    for (int step = step_begin;;) {
-        if (step + 1 >= step_end) {
-            compute(opA, 0);
-            break;
-        }
-        mfma_load_step<NB>(opB, p, step + 1, kb, wcol4, acol2);
-        x_fetch(step + 1);
-        compute(opA, 0);
-        x_publish(1);
+    // rounds of 8 steps, one per wave; the next round's sign words are already in
+    // flight while the activations are staged
+    MfmaOperands<NB> ops;
+    for (int r0 = step_begin; r0 < step_end; r0 += kMfmaWaves) {
+        const int step = r0 + wave;
+        const bool live = step < step_end;
+        mfma_load_step<NB>(ops, p, min(step, p.nsets - 1), kb, wcol4, acol2);
+        __syncthreads();  // previous round's readers are done with xs
+        stage_round(r0);
         __syncthreads();
-        ++step;
-        if (step + 1 >= step_end) {
-            compute(opB, 1);
-            break;
-        }
-        mfma_load_step<NB>(opA, p, step + 1, kb, wcol4, acol2);
-        x_fetch(step + 1);
-        compute(opB, 1);
-        x_publish(0);
-        __syncthreads();
-        ++step;
+        if (live) compute(ops);
     }
 
-    // ---- write: lane holds, for rows m = m0 + 16*mt + li, outputs n_base + 16*kb + 4*r + e ----
+    // ---- the 8 waves' accumulators meet in LDS -----------------------------------
+    __syncthreads();
+    float *red = (float *)xs;  // [wave][e*MT*4 + mt*4 + r][lane]
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt) {
+    for (int e = 0; e < 4; ++e)
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+                red[(wave * (16 * MT) + (e * MT + mt) * 4 + r) * 64 + lane] = acc[e][mt][r];
+    __syncthreads();
+    // thread (wave, lane) finishes values j = wave, wave + 8, ... of lane `lane`
+    for (int j = wave; j < 16 * MT; j += kMfmaWaves) {
+        float v = 0.0f;
+#pragma unroll
+        for (int w = 0; w < kMfmaWaves; ++w) v += red[(w * (16 * MT) + j) * 64 + lane];
+        const int e = j / (4 * MT), mt = (j / 4) % MT, r = j & 3;
         const int m = m0 + 16 * mt + li;
-        if (m >= p.M) continue;
+        const int n = n_base + 16 * kb + 4 * r + e;
+        if (m >= p.M || n >= p.N) continue;
         __half *out = p.out + (size_t)m * p.N;
+        if (p.ksplit == 1) {
+            out[n] = __float2half_rn(__half2float(out[n]) + v);
+            continue;
+        }
         unsigned long long *accum = p.accum + (size_t)m * p.N;
-#pragma unroll
-        for (int r = 0; r < 4; ++r)
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                const int n = n_base + 16 * kb + 4 * r + e;
-                if (n >= p.N) continue;
-                float v = acc[e][mt][r];
-                if (p.ksplit == 1) {
-                    out[n] = __float2half_rn(__half2float(out[n]) + v);
-                    continue;
-                }
-                v = (v == v) ? v : 65536.0f;
-                v = fminf(fmaxf(v, -65536.0f), 65536.0f);
-                const long long fx = __double2ll_rn((double)v * 4294967296.0);
-                const unsigned long long contrib = (unsigned long long)(fx + kBias) + kCountOne;
-                const unsigned long long old =
-                    __hip_atomic_fetch_add(accum + n, contrib, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                if ((int)(old >> 56) != p.ksplit - 1) continue;
-                const long long total = (long long)((old + contrib) & kSumMask) - (long long)p.ksplit * kBias;
-                const float y = (float)((double)total * (1.0 / 4294967296.0));
-                out[n] = __float2half_rn(__half2float(out[n]) + y);
-                __hip_atomic_store(accum + n, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            }
+        v = (v == v) ? v : 65536.0f;
+        v = fminf(fmaxf(v, -65536.0f), 65536.0f);
+        const long long fx = __double2ll_rn((double)v * 4294967296.0);
+        const unsigned long long contrib = (unsigned long long)(fx + kBias) + kCountOne;
+        const unsigned long long old =
+            __hip_atomic_fetch_add(accum + n, contrib, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if ((int)(old >> 56) != p.ksplit - 1) continue;
+        const long long total = (long long)((old + contrib) & kSumMask) - (long long)p.ksplit * kBias;
+        const float y = (float)((double)total * (1.0 / 4294967296.0));
+        out[n] = __float2half_rn(__half2float(out[n]) + y);
+        __hip_atomic_store(accum + n, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
 }
-
 
 __global__ void __launch_bounds__(256) copy_kernel(u32x4 *dst, const u32x4 *src, size_t n16)
 {
@@ -1046,11 +1039,15 @@ int run_mfma(Problem &p, hipStream_t stream)
     p.n_tiles = (p.N + kMfmaTileCols - 1) / kMfmaTileCols;
     p.mchunks = (p.M + 16 * mt - 1) / (16 * mt);
     p.nsets = p.K / kMfmaStepK;  // K-steps
-    long want = (long)target_blocks() * 2 / ((long)p.n_tiles * p.mchunks);
+    // K is already split 8 ways inside a workgroup; split it across workgroups only
+    // as far as needed to have about one workgroup per CU
+    long want = 256 / ((long)p.n_tiles * p.mchunks);
     if (want < 1) want = 1;
-    if (want > p.nsets) want = p.nsets;
+    if (want > p.nsets / kMfmaWaves) want = p.nsets / kMfmaWaves;
+    if (want < 1) want = 1;
     if (want > kMaxKSplit) want = kMaxKSplit;
     p.sets_per_split = (p.nsets + (int)want - 1) / (int)want;
+    p.sets_per_split = (p.sets_per_split + kMfmaWaves - 1) / kMfmaWaves * kMfmaWaves;  // whole rounds
     p.ksplit = (p.nsets + p.sets_per_split - 1) / p.sets_per_split;
     p.n_blocks = p.n_tiles * p.ksplit * p.mchunks;
     if (p.ksplit > 1) {
