@@ -150,6 +150,39 @@ int lutgemm_copy_bytes(void *dst, const void *src, size_t bytes, void *stream);
  * device (optional; they otherwise live until the process ends). */
 int lutgemm_release_workspaces(void);
 
+/*
+ * ---- decode-step glue (no counterpart in the reference) ----------------------
+ * The reference times token-by-token decoding through an eager framework model
+ * (model/opt.py:367-423); around each LUT-GEMV that costs some forty small
+ * framework kernels per decoder block.  These three entry points replace them,
+ * so that a block is eight launches.  fp16 tensors, row-major, contiguous.
+ */
+
+/* y[r] = fp16(fp16(x[r] * rsqrt(mean(x[r]^2) + eps)) * weight), r < rows;
+ * hidden % 8 == 0.  The same launch also zero-fills `clear_bytes` (multiple of
+ * 16, may be 0) at `clear`: the accumulate-into outputs of the GEMVs that
+ * consume y.  x, weight, y, clear 16-byte aligned. */
+int lutgemm_decode_rmsnorm_f16(const void *x, const void *weight, void *y, int rows, int hidden, float eps,
+                               void *clear, size_t clear_bytes, void *stream);
+
+/* One new token per sequence: rotary embedding of q and k at position
+ * *position (rotate-half convention: cos/sin tables [max_positions][head_dim],
+ * the two halves of a row equal), append k and v to the caches
+ * [batch][kv_heads][max_positions][head_dim], softmax(q k^T / sqrt(head_dim))
+ * v over cache positions 0..*position.  q [batch][heads*head_dim], k and v
+ * [batch][kv_heads*head_dim], out [batch][heads*head_dim]; heads a multiple of
+ * kv_heads; head_dim a multiple of 8, at most 256; max_positions at most 8192.
+ * `position` is a DEVICE pointer so that a captured graph can be replayed for
+ * successive tokens. */
+int lutgemm_decode_attention_f16(const void *q, const void *k, const void *v, const void *cos_table,
+                                 const void *sin_table, void *k_cache, void *v_cache, const int64_t *position,
+                                 void *out, int batch, int heads, int kv_heads, int head_dim, int max_positions,
+                                 void *stream);
+
+/* out = fp16(fp16(silu(gate)) * up) over `count` values (multiple of 8);
+ * pointers 16-byte aligned. */
+int lutgemm_decode_silu_mul_f16(const void *gate, const void *up, void *out, size_t count, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

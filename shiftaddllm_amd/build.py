@@ -45,13 +45,26 @@ def _run(cmd):
     subprocess.check_call(cmd)
 
 
+KERNEL_SOURCES = ("lutgemm_kernels.hip", "decode_kernels.hip")
+
+
 def build_kernel_library(force: bool = False) -> str:
-    src = os.path.join(CSRC, "lutgemm_kernels.hip")
-    hdr = os.path.join(INCLUDE, "lutgemm_gfx950.h")
-    if not force and _newer(KERNEL_LIB, src, hdr):
-        return KERNEL_LIB
+    """One object per source (only stale ones are recompiled), linked into the library."""
+    hdrs = [os.path.join(INCLUDE, "lutgemm_gfx950.h"), os.path.join(CSRC, "lutgemm_internal.h")]
     hipcc = os.path.join(ROCM, "bin", "hipcc")
-    _run([hipcc, *HIPCC_FLAGS, "-I", INCLUDE, "-o", KERNEL_LIB, src])
+    obj_dir = os.path.join(CSRC, "build")
+    os.makedirs(obj_dir, exist_ok=True)
+    flags = [f for f in HIPCC_FLAGS if f != "-shared"]
+    objs, relink = [], force or not os.path.exists(KERNEL_LIB)
+    for name in KERNEL_SOURCES:
+        src = os.path.join(CSRC, name)
+        obj = os.path.join(obj_dir, os.path.splitext(name)[0] + ".o")
+        if force or not _newer(obj, src, *hdrs):
+            _run([hipcc, *flags, "-I", INCLUDE, "-c", "-o", obj, src])
+            relink = True
+        objs.append(obj)
+    if relink or not _newer(KERNEL_LIB, *objs):
+        _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", KERNEL_LIB, *objs])
     return KERNEL_LIB
 
 

@@ -49,6 +49,7 @@
 #include <utility>
 
 #include "lutgemm_gfx950.h"
+#include "lutgemm_internal.h"
 
 namespace {
 
@@ -1093,6 +1094,8 @@ int run(int mode, const uint32_t *bW, const void *alpha, const void *qbias, cons
 }
 
 }  // namespace
+
+int lutgemm_internal_hip_fail(int hip_error) { return hip_fail((hipError_t)hip_error); }
 
 extern "C" {
 

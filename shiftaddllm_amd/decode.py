@@ -14,6 +14,12 @@ seven linears per block are LutLinear modules with a per-linear bit width taken
 from a `{"<module>": {"bits": b, ...}}` map (the schema of the reference's
 --quant_config files, model/opt.py:83-88).  One decode step can be captured in a
 HIP graph; q/k/v and gate/up can be issued as one fused launch each.
+
+Two implementations of everything between the linears exist: glue="hip" (the
+default) runs this library's fused kernels -- RMSNorm, rotary + KV append +
+attention, SiLU*up -- and lets o_proj / down_proj accumulate straight into the
+residual stream, eight launches per block; glue="torch" spells the same step in
+framework operations and is what the parity test's dense model is built from.
 """
 from __future__ import annotations
 
@@ -92,9 +98,11 @@ class LutDecoder(nn.Module):
 
     def __init__(self, cfg: DecoderConfig, quant_config: dict | None = None, batch: int = 1, seed: int = 0,
                  device="cuda:0", default_bits: int = 3, fuse_launches: bool = True,
-                 module_prefix: str = "model.layers"):
+                 module_prefix: str = "model.layers", glue: str = "hip"):
         super().__init__()
-        self.cfg, self.batch, self.fuse = cfg, batch, fuse_launches
+        if glue not in ("hip", "torch"):
+            raise ValueError(f"glue must be 'hip' or 'torch', got {glue!r}")
+        self.cfg, self.batch, self.fuse, self.glue = cfg, batch, fuse_launches, glue
         dev = torch.device(device)
         gen = torch.Generator(device=dev).manual_seed(seed)
         names = ("self_attn.q_proj", "self_attn.k_proj", "self_attn.v_proj", "self_attn.o_proj",
@@ -122,6 +130,15 @@ class LutDecoder(nn.Module):
         self.register_buffer("pos", torch.zeros((1,), dtype=torch.long, device=dev), persistent=False)
         self.register_buffer("logits", torch.zeros((batch, cfg.vocab_size), dtype=torch.float16, device=dev),
                              persistent=False)
+        # static activations of the glue="hip" step
+        H, KV, I = cfg.heads * hd, cfg.kv_heads * hd, cfg.intermediate
+        f16 = dict(dtype=torch.float16, device=dev)
+        self.register_buffer("x_res", torch.zeros((batch, cfg.hidden), **f16), persistent=False)
+        self.register_buffer("h_norm", torch.zeros((batch, cfg.hidden), **f16), persistent=False)
+        self.register_buffer("qkv", torch.zeros((batch * (H + 2 * KV),), **f16), persistent=False)
+        self.register_buffer("att", torch.zeros((batch, H), **f16), persistent=False)
+        self.register_buffer("gate_up", torch.zeros((2 * batch * I,), **f16), persistent=False)
+        self.register_buffer("act", torch.zeros((batch, I), **f16), persistent=False)
         self._graph = None
         self._stream = None
 
@@ -153,6 +170,62 @@ class LutDecoder(nn.Module):
     @torch.no_grad()
     def step(self):
         """Consumes self.ids [B] at position self.pos [1]; writes self.logits [B, V]."""
+        if self.glue == "hip":
+            return self._step_hip()
+        return self._step_torch()
+
+    def _gemv_into(self, lins, x, outs, sp):
+        """outs[i] += lins[i](x); one grouped launch when fusing."""
+        lib, B = native.cabi(), x.shape[0]
+        if self.fuse and len(lins) > 1:
+            arr = (native.RowwiseProblem * len(lins))()
+            for i, (l, o) in enumerate(zip(lins, outs)):
+                arr[i] = native.RowwiseProblem(l.binaryWeight.data_ptr(), l.alpha.data_ptr(), x.data_ptr(),
+                                               o.data_ptr(), l.N, l.K, l.wbit, l.num_groups, B)
+            rc = lib.lutgemm_gemv_rowwise_f16_grouped(len(lins), arr, sp)
+            if rc:
+                raise RuntimeError(lib.lutgemm_strerror(rc).decode())
+            return
+        for l, o in zip(lins, outs):
+            rc = lib.lutgemm_gemv_rowwise_f16(l.binaryWeight.data_ptr(), l.alpha.data_ptr(), x.data_ptr(),
+                                              o.data_ptr(), l.N, l.K, l.wbit, l.num_groups, B, sp)
+            if rc:
+                raise RuntimeError(lib.lutgemm_strerror(rc).decode())
+
+    def _step_hip(self):
+        cfg, B = self.cfg, self.batch
+        hd, H, KV, I = cfg.head_dim, cfg.heads, cfg.kv_heads, cfg.intermediate
+        lib = native.cabi()
+        sp = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+        def check(rc):
+            if rc:
+                raise RuntimeError(lib.lutgemm_strerror(rc).decode())
+
+        nq, nkv = B * H * hd, B * KV * hd
+        q, k, v = self.qkv[:nq], self.qkv[nq:nq + nkv], self.qkv[nq + nkv:]
+        g, u = self.gate_up[:B * I], self.gate_up[B * I:]
+        x, h = self.x_res, self.h_norm
+        torch.index_select(self.embed, 0, self.ids, out=x)
+        for li, blk in enumerate(self.blocks):
+            check(lib.lutgemm_decode_rmsnorm_f16(x.data_ptr(), blk.input_norm.data_ptr(), h.data_ptr(), B, cfg.hidden,
+                                                 cfg.rms_eps, self.qkv.data_ptr(), self.qkv.numel() * 2, sp))
+            self._gemv_into([blk.q_proj, blk.k_proj, blk.v_proj], h, [q, k, v], sp)
+            check(lib.lutgemm_decode_attention_f16(q.data_ptr(), k.data_ptr(), v.data_ptr(), self.cos.data_ptr(),
+                                                   self.sin.data_ptr(), self.k_cache[li].data_ptr(),
+                                                   self.v_cache[li].data_ptr(), self.pos.data_ptr(),
+                                                   self.att.data_ptr(), B, H, KV, hd, cfg.max_positions, sp))
+            self._gemv_into([blk.o_proj], self.att, [x], sp)            # x += o_proj(att)
+            check(lib.lutgemm_decode_rmsnorm_f16(x.data_ptr(), blk.post_norm.data_ptr(), h.data_ptr(), B, cfg.hidden,
+                                                 cfg.rms_eps, self.gate_up.data_ptr(), self.gate_up.numel() * 2, sp))
+            self._gemv_into([blk.gate_proj, blk.up_proj], h, [g, u], sp)
+            check(lib.lutgemm_decode_silu_mul_f16(g.data_ptr(), u.data_ptr(), self.act.data_ptr(), B * I, sp))
+            self._gemv_into([blk.down_proj], self.act, [x], sp)         # x += down_proj(act)
+        check(lib.lutgemm_decode_rmsnorm_f16(x.data_ptr(), self.final_norm.data_ptr(), h.data_ptr(), B, cfg.hidden,
+                                             cfg.rms_eps, None, 0, sp))
+        torch.matmul(h, self.lm_head.t(), out=self.logits)
+
+    def _step_torch(self):
         cfg, B = self.cfg, self.batch
         hd, H, KV = cfg.head_dim, cfg.heads, cfg.kv_heads
         x = self.embed[self.ids]                                    # [B, hidden]

@@ -29,6 +29,9 @@ C_ABI_SYMBOLS = (
     "lutgemm_algorithmic_bytes",
     "lutgemm_copy_bytes",
     "lutgemm_release_workspaces",
+    "lutgemm_decode_rmsnorm_f16",
+    "lutgemm_decode_attention_f16",
+    "lutgemm_decode_silu_mul_f16",
 )
 
 
@@ -98,6 +101,12 @@ def cabi() -> ctypes.CDLL:
         lib.lutgemm_copy_bytes.restype = ci
         lib.lutgemm_release_workspaces.argtypes = []
         lib.lutgemm_release_workspaces.restype = ci
+        lib.lutgemm_decode_rmsnorm_f16.argtypes = [vp, vp, vp, ci, ci, ctypes.c_float, vp, sz, vp]
+        lib.lutgemm_decode_rmsnorm_f16.restype = ci
+        lib.lutgemm_decode_attention_f16.argtypes = [vp] * 9 + [ci] * 5 + [vp]
+        lib.lutgemm_decode_attention_f16.restype = ci
+        lib.lutgemm_decode_silu_mul_f16.argtypes = [vp, vp, vp, sz, vp]
+        lib.lutgemm_decode_silu_mul_f16.restype = ci
         _cabi = lib
     return _cabi
 

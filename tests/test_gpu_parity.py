@@ -441,7 +441,7 @@ def test_decoder_matches_dense_dequantised_model(gpu_device):
     bits = sorted({l.wbit for b in lut.blocks for l in (b.q_proj, b.k_proj, b.down_proj, b.gate_proj)})
     assert len(bits) >= 2                                   # the draw really mixes bit widths
 
-    dense = decode.LutDecoder(cfg, qc, batch=2, seed=5, device=gpu_device, fuse_launches=False)
+    dense = decode.LutDecoder(cfg, qc, batch=2, seed=5, device=gpu_device, fuse_launches=False, glue="torch")
     table = {}
     for blk in dense.blocks:
         for lin in (blk.q_proj, blk.k_proj, blk.v_proj, blk.o_proj, blk.gate_proj, blk.up_proj, blk.down_proj):
@@ -455,7 +455,12 @@ def test_decoder_matches_dense_dequantised_model(gpu_device):
     lut.fuse = False
     lut._graph = None
     got_plain = run(lut, capture=False)
-    for name, got in (("fused", got_fused), ("graph", got_graph), ("plain", got_plain)):
+    # the same LutLinear layers between framework operations instead of the fused glue kernels
+    lut.glue, lut.fuse = "torch", True
+    got_torch_glue = run(lut, capture=False)
+    lut.glue = "hip"
+    for name, got in (("fused", got_fused), ("graph", got_graph), ("plain", got_plain),
+                      ("torch glue", got_torch_glue)):
         rel, mad = orc.error_metrics(got.numpy(), want.numpy())
         assert rel <= REL_L2_BAR and mad <= MAX_ABS_BAR, (name, rel, mad)
     # replaying the graph gives what the eager fused path gave
