@@ -199,6 +199,139 @@ attention_kernel(const __half *__restrict__ q, const __half *__restrict__ k, con
     }
 }
 
+// The same for head_dim HD in {64, 128}, with the memory latency taken in
+// parallel: a thread fetches the whole key row of its position before using it,
+// and the value rows are walked by 256/(HD/8) position groups with four rows in
+// flight per thread.  Dynamic LDS: (3*HD + max_pos + 4 + (256/(HD/8))*HD) floats.
+template <int HD>
+__global__ void __launch_bounds__(kThreads)
+attention_hd_kernel(const __half *__restrict__ q, const __half *__restrict__ k, const __half *__restrict__ v,
+                    const __half *__restrict__ cos_t, const __half *__restrict__ sin_t,
+                    __half *__restrict__ k_cache, __half *__restrict__ v_cache,
+                    const long long *__restrict__ pos_ptr, __half *__restrict__ out, int H, int KV, int max_pos)
+{
+    constexpr int kChunks = HD / 8;             // 16-byte chunks of a row
+    constexpr int kPosGroups = kThreads / kChunks;
+    extern __shared__ float lds[];
+    float *q_s = lds;
+    float *k_s = q_s + HD;
+    float *v_s = k_s + HD;
+    float *score = v_s + HD;
+    float *red = score + max_pos;
+    float *part = red + 4;
+
+    const int tid = threadIdx.x;
+    const int b = blockIdx.x / H, h = blockIdx.x % H;
+    const int rep = H / KV, kvh = h / rep;
+    int pos = (int)*pos_ptr;
+    pos = min(max(pos, 0), max_pos - 1);
+    const size_t cache_row0 = ((size_t)b * KV + kvh) * max_pos;
+
+    if (tid < HD) {
+        const int i = tid;
+        const float c = __half2float(cos_t[(size_t)pos * HD + i]);
+        const float s = __half2float(sin_t[(size_t)pos * HD + i]);
+        const __half *qh = q + ((size_t)b * H + h) * HD;
+        const __half *kh = k + ((size_t)b * KV + kvh) * HD;
+        const int j = i < HD / 2 ? i + HD / 2 : i - HD / 2;
+        const float sign = i < HD / 2 ? -1.0f : 1.0f;
+        const __half qr = __float2half_rn(__half2float(qh[i]) * c + sign * __half2float(qh[j]) * s);
+        const __half kr = __float2half_rn(__half2float(kh[i]) * c + sign * __half2float(kh[j]) * s);
+        const __half vv = v[((size_t)b * KV + kvh) * HD + i];
+        q_s[i] = __half2float(qr);
+        k_s[i] = __half2float(kr);
+        v_s[i] = __half2float(vv);
+        if (h % rep == 0) {
+            k_cache[(cache_row0 + pos) * HD + i] = kr;
+            v_cache[(cache_row0 + pos) * HD + i] = vv;
+        }
+    }
+    // key rows of earlier positions do not depend on the above: fetch before the barrier
+    const bool first_pass_cached = tid < pos;
+    u32x4 row[kChunks];
+    if (first_pass_cached) {
+        const u32x4 *src = (const u32x4 *)(k_cache + (cache_row0 + tid) * HD);
+#pragma unroll
+        for (int c = 0; c < kChunks; ++c) row[c] = src[c];
+    }
+    __syncthreads();
+
+    const float scale = rsqrtf((float)HD);
+    float local_max = -INFINITY;
+    for (int j = tid; j <= pos; j += kThreads) {
+        float dot = 0.0f;
+        if (j == pos) {
+#pragma unroll
+            for (int i = 0; i < HD; ++i) dot = fmaf(q_s[i], k_s[i], dot);
+        } else {
+            if (j != tid) {
+                const u32x4 *src = (const u32x4 *)(k_cache + (cache_row0 + j) * HD);
+#pragma unroll
+                for (int c = 0; c < kChunks; ++c) row[c] = src[c];
+            }
+#pragma unroll
+            for (int c = 0; c < kChunks; ++c) {
+                float f[8];
+                unpack8(row[c], f);
+#pragma unroll
+                for (int i = 0; i < 8; ++i) dot = fmaf(q_s[8 * c + i], f[i], dot);
+            }
+        }
+        dot *= scale;
+        score[j] = dot;
+        local_max = fmaxf(local_max, dot);
+    }
+    const float mx = block_reduce<true>(local_max, red);
+    float local_sum = 0.0f;
+    for (int j = tid; j <= pos; j += kThreads) {
+        const float e = __expf(score[j] - mx);
+        score[j] = e;
+        local_sum += e;
+    }
+    const float inv = 1.0f / block_reduce<false>(local_sum, red);  // its barriers also publish score[]
+
+    const int jg = tid / kChunks, ch = tid % kChunks;
+    float acc[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) acc[i] = 0.0f;
+    const u32x4 *vbase = (const u32x4 *)(v_cache + cache_row0 * HD) + ch;
+    int j = jg;
+    for (; j + 3 * kPosGroups < pos; j += 4 * kPosGroups) {
+        u32x4 r4[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) r4[u] = vbase[(size_t)(j + u * kPosGroups) * kChunks];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            float f[8];
+            unpack8(r4[u], f);
+            const float pj = score[j + u * kPosGroups];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) acc[i] = fmaf(pj, f[i], acc[i]);
+        }
+    }
+    for (; j < pos; j += kPosGroups) {
+        float f[8];
+        unpack8(vbase[(size_t)j * kChunks], f);
+        const float pj = score[j];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) acc[i] = fmaf(pj, f[i], acc[i]);
+    }
+    if (jg == 0) {
+        const float pj = score[pos];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) acc[i] = fmaf(pj, v_s[8 * ch + i], acc[i]);
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) part[jg * HD + 8 * ch + i] = acc[i];
+    __syncthreads();
+    if (tid < HD) {
+        float sum = 0.0f;
+#pragma unroll 8
+        for (int g = 0; g < kPosGroups; ++g) sum += part[g * HD + tid];
+        out[((size_t)b * H + h) * HD + tid] = __float2half_rn(sum * inv);
+    }
+}
+
 // out = fp16(fp16(silu(gate)) * up), 8 values per thread
 __global__ void __launch_bounds__(kThreads)
 silu_mul_kernel(const u32x4 *__restrict__ gate, const u32x4 *__restrict__ up, u32x4 *__restrict__ out, long units)
@@ -257,7 +390,25 @@ int lutgemm_decode_attention_f16(const void *q, const void *k, const void *v, co
     if (batch < 1 || heads < 1 || kv_heads < 1 || heads % kv_heads != 0) return LUTGEMM_EINVAL;
     if (head_dim < 8 || head_dim > kThreads || head_dim % 8 != 0) return LUTGEMM_EINVAL;
     if (max_positions < 1 || max_positions > 8192) return LUTGEMM_EINVAL;
-    if (!aligned16(k_cache)) return LUTGEMM_EALIGN;
+    if (!aligned16(k_cache) || !aligned16(v_cache)) return LUTGEMM_EALIGN;
+    if (head_dim == 64 || head_dim == 128) {
+        const int pos_groups = kThreads / (head_dim / 8);
+        const size_t lds_hd =
+            sizeof(float) * ((size_t)3 * head_dim + max_positions + 4 + (size_t)pos_groups * head_dim);
+        if (head_dim == 128)
+            hipLaunchKernelGGL(attention_hd_kernel<128>, dim3((unsigned)(batch * heads)), dim3(kThreads), lds_hd,
+                               (hipStream_t)stream, (const __half *)q, (const __half *)k, (const __half *)v,
+                               (const __half *)cos_table, (const __half *)sin_table, (__half *)k_cache,
+                               (__half *)v_cache, (const long long *)position, (__half *)out, heads, kv_heads,
+                               max_positions);
+        else
+            hipLaunchKernelGGL(attention_hd_kernel<64>, dim3((unsigned)(batch * heads)), dim3(kThreads), lds_hd,
+                               (hipStream_t)stream, (const __half *)q, (const __half *)k, (const __half *)v,
+                               (const __half *)cos_table, (const __half *)sin_table, (__half *)k_cache,
+                               (__half *)v_cache, (const long long *)position, (__half *)out, heads, kv_heads,
+                               max_positions);
+        return launch_status();
+    }
     const int groups = kThreads / head_dim;
     const size_t lds = sizeof(float) * ((size_t)3 * head_dim + max_positions + 4 + (size_t)groups * head_dim);
     hipLaunchKernelGGL(attention_kernel, dim3((unsigned)(batch * heads)), dim3(kThreads), lds, (hipStream_t)stream,

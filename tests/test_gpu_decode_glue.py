@@ -1,0 +1,123 @@
+"""GPU tests of the decode-step glue kernels, called through the C ABI and checked
+against plain fp32 torch restatements of the same operations."""
+import ctypes
+import math
+
+import pytest
+import torch
+
+from shiftaddllm_amd import native
+
+pytestmark = pytest.mark.gpu
+
+
+def _sp():
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _ok(rc):
+    assert rc == 0, native.cabi().lutgemm_strerror(rc).decode()
+
+
+@pytest.mark.parametrize("rows,hidden", [(1, 4096), (8, 4096), (3, 264), (2, 11008)])
+def test_rmsnorm_and_clear(gpu_device, rows, hidden):
+    lib = native.cabi()
+    g = torch.Generator(device=gpu_device).manual_seed(rows * 131 + hidden)
+    x = (torch.randn((rows, hidden), generator=g, device=gpu_device) * 3).half()
+    w = (1 + 0.1 * torch.randn((hidden,), generator=g, device=gpu_device)).half()
+    y = torch.empty_like(x)
+    junk = torch.full((rows * 3 * hidden + 8,), 7.0, dtype=torch.float16, device=gpu_device)
+    clear_bytes = (junk.numel() - 8) * 2
+    _ok(lib.lutgemm_decode_rmsnorm_f16(x.data_ptr(), w.data_ptr(), y.data_ptr(), rows, hidden, 1e-5,
+                                       junk.data_ptr(), clear_bytes, _sp()))
+    torch.cuda.synchronize()
+    xf = x.float()
+    want = (xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + 1e-5)).half().float() * w.float()
+    assert torch.allclose(y.float(), want, rtol=2e-3, atol=2e-3)
+    assert torch.count_nonzero(junk[:-8]) == 0 and torch.all(junk[-8:] == 7.0)   # cleared exactly the range
+
+
+def test_rmsnorm_rejects_bad_arguments(gpu_device):
+    lib = native.cabi()
+    x = torch.zeros((1, 64), dtype=torch.float16, device=gpu_device)
+    assert lib.lutgemm_decode_rmsnorm_f16(x.data_ptr(), x.data_ptr(), x.data_ptr(), 1, 60, 1e-5, None, 0, _sp()) == -1
+    assert lib.lutgemm_decode_rmsnorm_f16(x.data_ptr(), x.data_ptr(), x.data_ptr(), 1, 64, 1e-5, None, 16, _sp()) == -1
+    assert lib.lutgemm_decode_rmsnorm_f16(x.data_ptr() + 2, x.data_ptr(), x.data_ptr(), 1, 32, 1e-5, None, 0,
+                                          _sp()) == -2
+
+
+def _rope(t, cos, sin):
+    half = t.shape[-1] // 2
+    rot = torch.cat([-t[..., half:], t[..., :half]], dim=-1)
+    return t * cos + rot * sin
+
+
+@pytest.mark.parametrize("B,H,KV,hd,max_pos,positions", [
+    (1, 32, 32, 128, 256, (0, 1, 100, 255)),
+    (2, 4, 2, 64, 32, (0, 5, 31)),
+    (2, 8, 2, 128, 700, (0, 300, 699)),        # more keys than threads in a workgroup
+    (1, 4, 4, 96, 40, (0, 17, 39)),            # the generic head-dim path
+    (3, 6, 3, 64, 520, (519,)),
+])
+def test_attention_step(gpu_device, B, H, KV, hd, max_pos, positions):
+    lib = native.cabi()
+    g = torch.Generator(device=gpu_device).manual_seed(B * 1000 + H * 10 + hd)
+    inv = 1.0 / (10000.0 ** (torch.arange(0, hd, 2, device=gpu_device).float() / hd))
+    ang = torch.arange(max_pos, device=gpu_device).float()[:, None] * inv[None, :]
+    cos = torch.cat([ang.cos(), ang.cos()], -1).half()
+    sin = torch.cat([ang.sin(), ang.sin()], -1).half()
+    for pos in positions:
+        kc = torch.randn((B, KV, max_pos, hd), generator=g, device=gpu_device).half()
+        vc = torch.randn((B, KV, max_pos, hd), generator=g, device=gpu_device).half()
+        kc0, vc0 = kc.clone(), vc.clone()
+        q = torch.randn((B, H * hd), generator=g, device=gpu_device).half()
+        k = torch.randn((B, KV * hd), generator=g, device=gpu_device).half()
+        v = torch.randn((B, KV * hd), generator=g, device=gpu_device).half()
+        out = torch.zeros((B, H * hd), dtype=torch.float16, device=gpu_device)
+        p = torch.tensor([pos], dtype=torch.long, device=gpu_device)
+        _ok(lib.lutgemm_decode_attention_f16(q.data_ptr(), k.data_ptr(), v.data_ptr(), cos.data_ptr(),
+                                             sin.data_ptr(), kc.data_ptr(), vc.data_ptr(), p.data_ptr(),
+                                             out.data_ptr(), B, H, KV, hd, max_pos, _sp()))
+        torch.cuda.synchronize()
+        # fp32 restatement
+        c, s = cos[pos].float(), sin[pos].float()
+        qr = _rope(q.float().view(B, H, hd), c, s).half().float()
+        kr = _rope(k.float().view(B, KV, hd), c, s).half()
+        want_k, want_v = kc0.clone(), vc0.clone()
+        want_k[:, :, pos] = kr
+        want_v[:, :, pos] = v.view(B, KV, hd)
+        assert torch.equal(vc, want_v)
+        assert torch.allclose(kc.float(), want_k.float(), rtol=2e-3, atol=2e-3)
+        assert torch.equal(kc[:, :, pos + 1:], kc0[:, :, pos + 1:]) and torch.equal(kc[:, :, :pos], kc0[:, :, :pos])
+        keys = want_k[:, :, :pos + 1].float().repeat_interleave(H // KV, dim=1)       # [B, H, T, hd]
+        vals = want_v[:, :, :pos + 1].float().repeat_interleave(H // KV, dim=1)
+        att = torch.softmax(torch.einsum("bhd,bhtd->bht", qr, keys) / math.sqrt(hd), dim=-1)
+        want = torch.einsum("bht,bhtd->bhd", att, vals).reshape(B, H * hd)
+        assert torch.allclose(out.float(), want, rtol=5e-3, atol=5e-3), (pos, (out.float() - want).abs().max())
+
+
+def test_attention_rejects_bad_arguments(gpu_device):
+    lib = native.cabi()
+    t = torch.zeros((4096,), dtype=torch.float16, device=gpu_device)
+    p = torch.zeros((1,), dtype=torch.long, device=gpu_device)
+    a = t.data_ptr()
+    call = lambda B, H, KV, hd, mp: lib.lutgemm_decode_attention_f16(a, a, a, a, a, a, a, p.data_ptr(), a, B, H, KV,
+                                                                     hd, mp, _sp())
+    assert call(1, 4, 3, 64, 16) == -1        # heads not a multiple of kv heads
+    assert call(1, 4, 4, 60, 16) == -1        # head dim not a multiple of 8
+    assert call(1, 4, 4, 512, 16) == -1       # head dim too large
+    assert call(1, 4, 4, 64, 10000) == -1     # more positions than the kernel's LDS budget
+
+
+@pytest.mark.parametrize("count", [8, 11008, 8 * 11008, 4104])
+def test_silu_mul(gpu_device, count):
+    lib = native.cabi()
+    g = torch.Generator(device=gpu_device).manual_seed(count)
+    gate = (torch.randn((count,), generator=g, device=gpu_device) * 4).half()
+    up = torch.randn((count,), generator=g, device=gpu_device).half()
+    out = torch.empty_like(gate)
+    _ok(lib.lutgemm_decode_silu_mul_f16(gate.data_ptr(), up.data_ptr(), out.data_ptr(), count, _sp()))
+    torch.cuda.synchronize()
+    want = torch.nn.functional.silu(gate.float()).half().float() * up.float()
+    assert torch.allclose(out.float(), want, rtol=2e-3, atol=1e-3)
+    assert lib.lutgemm_decode_silu_mul_f16(gate.data_ptr(), up.data_ptr(), out.data_ptr(), count + 1, _sp()) == -1
