@@ -151,6 +151,37 @@ int lutgemm_copy_bytes(void *dst, const void *src, size_t bytes, void *stream);
 int lutgemm_release_workspaces(void);
 
 /*
+ * Row-wise GEMVs with the neighbouring element-wise work of a decoder block
+ * folded in (no counterpart in the reference, whose modules run them as
+ * separate framework kernels).  Up to LUTGEMM_MAX_GROUP problems per launch.
+ *   norm_weight_f16 : NULL, or fp16 [K]: the GEMV input is
+ *                     fp16(fp16(x * rsqrt(mean(x^2) + norm_eps)) * norm_weight)
+ *                     per row of x (RMSNorm), formed inside the kernel;
+ *   gate_f16        : NULL, or fp16 [M][K]: the GEMV input is
+ *                     fp16(fp16(silu(gate)) * x)  (SwiGLU);
+ *                     at most one of the two per problem; both 16-byte aligned;
+ *   overwrite       : 0 = out += y like every other entry point, 1 = out = y
+ *                     (out need not be initialised).
+ * A problem with none of the three is the plain row-wise GEMV.  The problems of
+ * one call must share their transform (all norm, all gate or all none;
+ * LUTGEMM_EUNSUP otherwise).  Problems with a transform or with overwrite run on
+ * the look-up kernel, whatever M.
+ */
+typedef struct lutgemm_fused_problem {
+    const uint32_t *bW;
+    const void *alpha_f16;
+    const void *x_f16;
+    void *out_f16;
+    int N, K, nb, num_groups, M;
+    int overwrite;
+    const void *norm_weight_f16;
+    const void *gate_f16;
+    float norm_eps;
+} lutgemm_fused_problem;
+
+int lutgemm_gemv_rowwise_f16_fused(int count, const lutgemm_fused_problem *problems, void *stream);
+
+/*
  * ---- decode-step glue (no counterpart in the reference) ----------------------
  * The reference times token-by-token decoding through an eager framework model
  * (model/opt.py:367-423); around each LUT-GEMV that costs some forty small

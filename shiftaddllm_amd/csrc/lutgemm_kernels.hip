@@ -112,6 +112,11 @@ struct Problem {
     int block_begin;     // grouped launches: first flat workgroup index of this problem
     int mchunks;         // activation rows are handled in chunks of MROWS
     int n_blocks;        // workgroups of this problem in the flat grid
+    // fused input transforms and output mode (row-wise look-up path only)
+    const __half *norm_w;  // non-null: the input is fp16(fp16(x * rsqrt(mean(x^2) + norm_eps)) * norm_w)
+    const __half *gate;    // non-null [M][K]: the input is fp16(fp16(silu(gate)) * x)
+    float norm_eps;
+    int overwrite;         // 1: out = y instead of out += y
 };
 
 // Flat workgroup index (relative to the problem) -> (tile, kslice, m).
@@ -250,17 +255,71 @@ __device__ __forceinline__ void stage_alpha(const SetOperands<NB, NSTEPS, MODE> 
 }
 
 // The 8 activations (fp16) of the chunk whose table this thread helps to build:
-// chunk tb of set `set` of activation row x.  Chunks beyond K read as zero.
-__device__ __forceinline__ u32x4 load_x_chunk(const Problem &p, const __half *x, int set, int tb)
+// chunk tb of set `set` of activation row x.  Fetching and finishing are separate
+// so that the loads stay in flight across the look-ups of the current item.
+// FUSED kernels also fetch the matching chunk of the norm weight or of the gate row.
+// compile-time input transform of a kernel instance
+constexpr int kXNone = 0, kXNorm = 1, kXGate = 2;
+
+struct XChunk {
+    u32x4 x, other;
+    int kc;     // first input of the chunk (clamped into the row)
+    bool live;  // chunks beyond K read as zero
+};
+
+template <int XF>
+__device__ __forceinline__ XChunk fetch_x_chunk(const Problem &p, const __half *x, const __half *gate, int set,
+                                                int tb)
 {
     const int k0 = (set * kTables + tb) * 8;
-    const u32x4 xr = *(const u32x4 *)(x + min(k0, p.K - 8));
-    const bool live = k0 < p.K;
+    const int kc = min(k0, p.K - 8);
+    XChunk c;
+    c.x = *(const u32x4 *)(x + kc);
+    c.other = (u32x4){0u, 0u, 0u, 0u};
+    // (the norm weight is read when the chunk is finished: every workgroup reads the
+    // same few KB, an L1/L2 hit, and four registers less are held across the look-ups)
+    if constexpr (XF == kXGate) c.other = *(const u32x4 *)(gate + kc);
+    c.kc = kc;
+    c.live = k0 < p.K;
+    return c;
+}
+
+// With a norm weight the chunk is scaled by `rscale` (the row's reciprocal RMS) and
+// the weight; with a gate row it is multiplied by silu(gate); both with the
+// roundings of the separate fp16 operations they replace.
+template <int XF>
+__device__ __forceinline__ u32x4 finish_x_chunk(const Problem &p, const XChunk &c, float rscale)
+{
+    u32x4 xr = c.x;
+    if constexpr (XF != kXNone) {
+        {
+            u32x4 other = c.other;
+            if constexpr (XF == kXNorm) other = *(const u32x4 *)(p.norm_w + c.kc);
+            const uint32_t a[4] = {c.x.x, c.x.y, c.x.z, c.x.w};
+            const uint32_t b[4] = {other.x, other.y, other.z, other.w};
+            uint32_t o[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                float v[2];
+#pragma unroll
+                for (int hh = 0; hh < 2; ++hh) {
+                    const float xv = half_bits_to_float((a[j] >> (16 * hh)) & 0xffffu);
+                    const float bv = half_bits_to_float((b[j] >> (16 * hh)) & 0xffffu);
+                    if constexpr (XF == kXGate)
+                        v[hh] = half_bits_to_float(float_to_half_bits(__fdividef(bv, 1.0f + __expf(-bv)))) * xv;
+                    else
+                        v[hh] = half_bits_to_float(float_to_half_bits(xv * rscale)) * bv;
+                }
+                o[j] = float_to_half_bits(v[0]) | (float_to_half_bits(v[1]) << 16);
+            }
+            xr = (u32x4){o[0], o[1], o[2], o[3]};
+        }
+    }
     u32x4 r;
-    r.x = live ? xr.x : 0u;
-    r.y = live ? xr.y : 0u;
-    r.z = live ? xr.z : 0u;
-    r.w = live ? xr.w : 0u;
+    r.x = c.live ? xr.x : 0u;
+    r.y = c.live ? xr.y : 0u;
+    r.z = c.live ? xr.z : 0u;
+    r.w = c.live ? xr.w : 0u;
     return r;
 }
 
@@ -380,7 +439,7 @@ __device__ __forceinline__ void lookup_set(const SetOperands<NB, NSTEPS, MODE> &
 // mchunk*MROWS .. +MROWS-1.  The sign words of a set are loaded once and used
 // for all MROWS rows; tables are built per (set, row) and double buffered, so the
 // work items of the pipeline are the (set, row) pairs in order.
-template <int NB, int NSTEPS, int MODE, int MROWS>
+template <int NB, int NSTEPS, int MODE, int MROWS, int XF = kXNone>
 __device__ __forceinline__ void gemv_tile(const Problem &p, int tile, int kslice, int mchunk, float *lut)
 {
     const int tid = threadIdx.x;
@@ -397,6 +456,10 @@ __device__ __forceinline__ void gemv_tile(const Problem &p, int tile, int kslice
     const __half *xrow[MROWS];
 #pragma unroll
     for (int r = 0; r < MROWS; ++r) xrow[r] = p.x + (size_t)min(m0 + r, p.M - 1) * p.K;
+    const __half *grow[MROWS];
+#pragma unroll
+    for (int r = 0; r < MROWS; ++r)
+        grow[r] = (XF == kXGate) ? p.gate + (size_t)min(m0 + r, p.M - 1) * p.K : nullptr;
 
     // per-lane look-up constants (see lookup_set)
     uint32_t lane_off = 0;
@@ -442,6 +505,22 @@ __device__ __forceinline__ void gemv_tile(const Problem &p, int tile, int kslice
     // set i+1 are in flight.  No register copies between them (a copy would have
     // to wait for the loads), and the has-next test is peeled out of the load
     // path so that the compiler can count the loads in flight exactly.
+    // fused RMSNorm: every workgroup forms the reciprocal RMS of its rows itself (K
+    // fp16 values per row, from L2).  The row is requested BEFORE the first sign
+    // words so that, loads returning in order, it can be waited for alone.
+    constexpr int kNormChunks = 2;  // 16-byte chunks per thread held in registers: K <= 8192
+    u32x4 nx[XF == kXNorm ? MROWS : 1][kNormChunks];
+    if constexpr (XF == kXNorm) {
+        {
+#pragma unroll
+            for (int r = 0; r < MROWS; ++r)
+#pragma unroll
+                for (int u = 0; u < kNormChunks; ++u)
+                    nx[r][u] = *(const u32x4 *)(xrow[r] + 8 * min(tid + kThreads * u, p.K / 8 - 1));
+        }
+    }
+    XChunk xc0 = fetch_x_chunk<XF>(p, xrow[0], grow[0], set_begin, tb);
+
     SetOperands<NB, NSTEPS, MODE> opA, opB;
     load_set<NB, NSTEPS, MODE>(opA, p, set_begin, kw, q, lc);
 
@@ -454,8 +533,46 @@ __device__ __forceinline__ void gemv_tile(const Problem &p, int tile, int kslice
         for (int s = 0; s < NSTEPS; ++s)
             out_raw[r][s] = *(const u32x2 *)((const char *)(p.out + (size_t)min(m0 + r, p.M - 1) * p.N) + lc.col2[s]);
 
+    float rscale[MROWS];
+#pragma unroll
+    for (int r = 0; r < MROWS; ++r) rscale[r] = 1.0f;
+    if constexpr (XF == kXNorm) {
+        {
+            float ss[MROWS];
+#pragma unroll
+            for (int r = 0; r < MROWS; ++r) {
+                ss[r] = 0.0f;
+                auto add_chunk = [&](const u32x4 &v) {
+                    const uint32_t w4[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        const float lo = half_bits_to_float(w4[j] & 0xffffu), hi = half_bits_to_float(w4[j] >> 16);
+                        ss[r] = fmaf(lo, lo, fmaf(hi, hi, ss[r]));
+                    }
+                };
+#pragma unroll
+                for (int u = 0; u < kNormChunks; ++u)
+                    if (tid + kThreads * u < p.K / 8) add_chunk(nx[r][u]);
+                for (int c = tid + kThreads * kNormChunks; c < p.K / 8; c += kThreads)  // K > 16384
+                    add_chunk(*(const u32x4 *)(xrow[r] + 8 * c));
+#pragma unroll
+                for (int off = 32; off > 0; off >>= 1) ss[r] += __shfl_xor(ss[r], off);
+                if (lane == 0) lut[wave * MROWS + r] = ss[r];
+            }
+            __syncthreads();
+#pragma unroll
+            for (int r = 0; r < MROWS; ++r) {
+                float t = 0.0f;
+#pragma unroll
+                for (int w = 0; w < kWaves; ++w) t += lut[w * MROWS + r];
+                rscale[r] = rsqrtf(t / (float)p.K + p.norm_eps);
+            }
+            __syncthreads();  // the tables are built over the same LDS words
+        }
+    }
+
     int buf = 0;
-    build_tables(load_x_chunk(p, xrow[0], set_begin, tb), lut, 0, tb, eb);
+    build_tables(finish_x_chunk<XF>(p, xc0, rscale[0]), lut, 0, tb, eb);
     stage_alpha<NB, NSTEPS, MODE>(opA, stage, 0, tid);
     __syncthreads();
     // Steady state, per (set, row) item: fetch the activations of the next item,
@@ -468,10 +585,10 @@ __device__ __forceinline__ void gemv_tile(const Problem &p, int tile, int kslice
 #pragma unroll
         for (int r = 0; r < MROWS; ++r) {
             const bool more = (r + 1 < MROWS) || decltype(has_next_set)::value;
-            u32x4 xn = (u32x4){0u, 0u, 0u, 0u};
+            XChunk xn{};
             if (more)
-                xn = (r + 1 < MROWS) ? load_x_chunk(p, xrow[(r + 1) % MROWS], set, tb)
-                                     : load_x_chunk(p, xrow[0], set + 1, tb);
+                xn = (r + 1 < MROWS) ? fetch_x_chunk<XF>(p, xrow[(r + 1) % MROWS], grow[(r + 1) % MROWS], set, tb)
+                                     : fetch_x_chunk<XF>(p, xrow[0], grow[0], set + 1, tb);
             // opaque to the optimiser: otherwise the 48 look-up addresses of a set are
             // kept in registers across all rows instead of being recomputed (1 op each)
             asm volatile("" : "+v"(lane_off));
@@ -480,7 +597,7 @@ __device__ __forceinline__ void gemv_tile(const Problem &p, int tile, int kslice
             if (more) {
                 buf ^= 1;
                 lane_off ^= kFlip;
-                build_tables(xn, lut, buf, tb, eb);
+                build_tables(finish_x_chunk<XF>(p, xn, rscale[(r + 1) % MROWS]), lut, buf, tb, eb);
                 if (r + 1 == MROWS) {  // moving on to the next set: its alphas go to the other stage buffer
                     abuf ^= 1;
                     stage_alpha<NB, NSTEPS, MODE>(nxt, stage, abuf, tid);
@@ -532,6 +649,7 @@ __device__ __forceinline__ void gemv_tile(const Problem &p, int tile, int kslice
                 const int n = n_lane + s * kStepCols;
                 if (n < p.N) {
                     u32x2 raw = out_raw[r][s];
+                    if (p.overwrite) raw = (u32x2){0u, 0u};
                     const float o0 = half_bits_to_float(raw.x & 0xffffu) + acc[r][s][0];
                     const float o1 = half_bits_to_float(raw.x >> 16) + acc[r][s][1];
                     const float o2 = half_bits_to_float(raw.y & 0xffffu) + acc[r][s][2];
@@ -576,8 +694,8 @@ __device__ __forceinline__ void gemv_tile(const Problem &p, int tile, int kslice
                 const long long total =
                     (long long)((old[s][i] + contrib[s][i]) & kSumMask) - (long long)p.ksplit * kBias;
                 const float y = (float)((double)total * (1.0 / 4294967296.0));
-                const float o = half_bits_to_float((raw2[i >> 1] >> (16 * (i & 1))) & 0xffffu) + y;
-                out[n + i] = __float2half_rn(o);
+                const float prev = p.overwrite ? 0.0f : half_bits_to_float((raw2[i >> 1] >> (16 * (i & 1))) & 0xffffu);
+                out[n + i] = __float2half_rn(prev + y);
                 __hip_atomic_store(accum + n + i, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             }
         }
@@ -595,8 +713,10 @@ __global__ void __launch_bounds__(kThreads) lut_gemv_kernel(const Problem p)
 
 // Several row-wise problems in one launch (flat 1-D grid).  Bit widths may
 // differ between the problems of a group.
-template <int NSTEPS>
-__global__ void __launch_bounds__(kThreads) lut_gemv_group_kernel(const Group g)
+// XF: the input transform shared by all problems of the launch.
+template <int NSTEPS, int XF>
+__global__ void __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4, 4)))
+lut_gemv_group_kernel(const Group g)
 {
     __shared__ __attribute__((aligned(16))) float lut[kLutDwords + kStageDwords];
     const int b = blockIdx.x;
@@ -608,10 +728,10 @@ __global__ void __launch_bounds__(kThreads) lut_gemv_group_kernel(const Group g)
     int tile, kslice, m;
     decode_block(p, b - p.block_begin, tile, kslice, m);
     switch (p.nb) {
-    case 1: gemv_tile<1, NSTEPS, kRowF16, 1>(p, tile, kslice, m, lut); break;
-    case 2: gemv_tile<2, NSTEPS, kRowF16, 1>(p, tile, kslice, m, lut); break;
-    case 3: gemv_tile<3, NSTEPS, kRowF16, 1>(p, tile, kslice, m, lut); break;
-    default: gemv_tile<4, NSTEPS, kRowF16, 1>(p, tile, kslice, m, lut); break;
+    case 1: gemv_tile<1, NSTEPS, kRowF16, 1, XF>(p, tile, kslice, m, lut); break;
+    case 2: gemv_tile<2, NSTEPS, kRowF16, 1, XF>(p, tile, kslice, m, lut); break;
+    case 3: gemv_tile<3, NSTEPS, kRowF16, 1, XF>(p, tile, kslice, m, lut); break;
+    default: gemv_tile<4, NSTEPS, kRowF16, 1, XF>(p, tile, kslice, m, lut); break;
     }
 }
 
@@ -1093,6 +1213,86 @@ int run(int mode, const uint32_t *bW, const void *alpha, const void *qbias, cons
     }
 }
 
+// Up to kMaxGroup row-wise problems in one launch of the look-up kernel.  Problems
+// with enough rows for the matrix-core kernel (and no fused transform) are launched
+// one by one on that path instead.
+int run_group(int count, const lutgemm_fused_problem *problems, hipStream_t stream)
+{
+    Group g{};
+    g.count = count;
+    size_t words = 0;
+    long total_bytes = 0;
+    bool plain = true, all_mfma = true;
+    int xform = kXNone;
+    for (int i = 0; i < count; ++i) {
+        const lutgemm_fused_problem &q = problems[i];
+        Problem &p = g.p[i];
+        int rc = fill_problem(p, kRowF16, q.bW, q.alpha_f16, nullptr, q.x_f16, q.out_f16, q.N, q.K, q.nb,
+                              q.num_groups, q.M);
+        if (rc != LUTGEMM_OK) return rc;
+        if (q.norm_weight_f16 && q.gate_f16) return LUTGEMM_EINVAL;
+        if (q.overwrite != 0 && q.overwrite != 1) return LUTGEMM_EINVAL;
+        if (q.norm_weight_f16 && !(q.norm_eps >= 0.0f)) return LUTGEMM_EINVAL;
+        if (!aligned(q.norm_weight_f16, 16) || !aligned(q.gate_f16, 16)) return LUTGEMM_EALIGN;
+        p.norm_w = (const __half *)q.norm_weight_f16;
+        p.gate = (const __half *)q.gate_f16;
+        p.norm_eps = q.norm_eps;
+        p.overwrite = q.overwrite;
+        // one kernel instance per transform: the problems of a launch share theirs
+        const int mine = p.norm_w ? kXNorm : p.gate ? kXGate : kXNone;
+        if (i > 0 && mine != xform) return LUTGEMM_EUNSUP;
+        xform = mine;
+        plain = plain && !p.norm_w && !p.gate && !p.overwrite;
+        all_mfma = all_mfma && mfma_eligible(p, kRowF16);
+        words += (size_t)q.M * q.N;
+        total_bytes += (long)q.N * (q.K / 8) * q.nb * q.M;
+    }
+    if (plain && all_mfma) {
+        for (int i = 0; i < count; ++i) {
+            int rc = run_mfma(g.p[i], stream);
+            if (rc != LUTGEMM_OK) return rc;
+        }
+        return LUTGEMM_OK;
+    }
+    // Share the launch's workgroup budget in proportion to each problem's sign
+    // bytes.  The budget is what is resident at once (two workgroups on each of 256
+    // CUs): a launch a little above it runs a second, mostly empty round that costs
+    // as much as the first (3 x 4096x4096: 15.6 us with 768 workgroups, 10.8 with 384).
+    const long budget = (long)target_blocks();
+    int begin = 0;
+    bool any_split = false;
+    for (int i = 0; i < count; ++i) {
+        Problem &p = g.p[i];
+        const long mine = (long)p.N * (p.K / 8) * p.nb * p.M;
+        long want = budget * mine / (total_bytes > 0 ? total_bytes : 1);
+        if (want < 1) want = 1;
+        plan_problem(p, 1, 1, want);
+        p.block_begin = begin;
+        begin += p.n_blocks;
+        any_split = any_split || p.ksplit > 1;
+    }
+    if (any_split) {
+        unsigned long long *base = nullptr;
+        int rc = get_workspace(stream, words, &base);
+        if (rc != LUTGEMM_OK) return rc;
+        size_t off = 0;
+        for (int i = 0; i < count; ++i) {
+            g.p[i].accum = base + off;
+            off += (size_t)g.p[i].M * g.p[i].N;
+        }
+    }
+    const dim3 grid((unsigned)begin), block(kThreads);
+    if (xform == kXNorm)
+        hipLaunchKernelGGL((lut_gemv_group_kernel<1, kXNorm>), grid, block, 0, stream, g);
+    else if (xform == kXGate)
+        hipLaunchKernelGGL((lut_gemv_group_kernel<1, kXGate>), grid, block, 0, stream, g);
+    else
+        hipLaunchKernelGGL((lut_gemv_group_kernel<1, kXNone>), grid, block, 0, stream, g);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return hip_fail(e);
+    return LUTGEMM_OK;
+}
+
 }  // namespace
 
 int lutgemm_internal_hip_fail(int hip_error) { return hip_fail((hipError_t)hip_error); }
@@ -1127,47 +1327,26 @@ int lutgemm_gemv_rowwise_f16_grouped(int count, const lutgemm_rowwise_problem *p
                                      void *stream_v)
 {
     if (!problems || count < 1 || count > kMaxGroup) return LUTGEMM_EINVAL;
-    Group g{};
-    g.count = count;
-    hipStream_t stream = (hipStream_t)stream_v;
-    size_t words = 0;
-    long total_bytes = 0;
+    lutgemm_fused_problem f[kMaxGroup] = {};
     for (int i = 0; i < count; ++i) {
         const lutgemm_rowwise_problem &q = problems[i];
-        int rc = fill_problem(g.p[i], kRowF16, q.bW, q.alpha_f16, nullptr, q.x_f16, q.out_f16, q.N,
-                              q.K, q.nb, q.num_groups, q.M);
-        if (rc != LUTGEMM_OK) return rc;
-        words += (size_t)q.M * q.N;
-        total_bytes += (long)q.N * (q.K / 8) * q.nb * q.M;
+        f[i].bW = q.bW;
+        f[i].alpha_f16 = q.alpha_f16;
+        f[i].x_f16 = q.x_f16;
+        f[i].out_f16 = q.out_f16;
+        f[i].N = q.N;
+        f[i].K = q.K;
+        f[i].nb = q.nb;
+        f[i].num_groups = q.num_groups;
+        f[i].M = q.M;
     }
-    // share the launch's workgroup budget in proportion to each problem's sign bytes
-    const long budget = (long)target_blocks() * (count > 1 ? 2 : 1);
-    int begin = 0;
-    bool any_split = false;
-    for (int i = 0; i < count; ++i) {
-        Problem &p = g.p[i];
-        const long mine = (long)p.N * (p.K / 8) * p.nb * p.M;
-        long want = budget * mine / (total_bytes > 0 ? total_bytes : 1);
-        if (want < 1) want = 1;
-        plan_problem(p, 1, 1, want);
-        p.block_begin = begin;
-        begin += p.n_blocks;
-        any_split = any_split || p.ksplit > 1;
-    }
-    if (any_split) {
-        unsigned long long *base = nullptr;
-        int rc = get_workspace(stream, words, &base);
-        if (rc != LUTGEMM_OK) return rc;
-        size_t off = 0;
-        for (int i = 0; i < count; ++i) {
-            g.p[i].accum = base + off;
-            off += (size_t)g.p[i].M * g.p[i].N;
-        }
-    }
-    hipLaunchKernelGGL((lut_gemv_group_kernel<1>), dim3((unsigned)begin), dim3(kThreads), 0, stream, g);
-    hipError_t e = hipGetLastError();
-    if (e != hipSuccess) return hip_fail(e);
-    return LUTGEMM_OK;
+    return run_group(count, f, (hipStream_t)stream_v);
+}
+
+int lutgemm_gemv_rowwise_f16_fused(int count, const lutgemm_fused_problem *problems, void *stream_v)
+{
+    if (!problems || count < 1 || count > kMaxGroup) return LUTGEMM_EINVAL;
+    return run_group(count, problems, (hipStream_t)stream_v);
 }
 
 int lutgemm_gemv_uniform_f16(const uint32_t *bW, const void *alpha_f16, const void *qbias_f16,

@@ -103,6 +103,7 @@ class LutDecoder(nn.Module):
         if glue not in ("hip", "torch"):
             raise ValueError(f"glue must be 'hip' or 'torch', got {glue!r}")
         self.cfg, self.batch, self.fuse, self.glue = cfg, batch, fuse_launches, glue
+        self.fold_norm = True
         dev = torch.device(device)
         gen = torch.Generator(device=dev).manual_seed(seed)
         names = ("self_attn.q_proj", "self_attn.k_proj", "self_attn.v_proj", "self_attn.o_proj",
@@ -192,6 +193,20 @@ class LutDecoder(nn.Module):
             if rc:
                 raise RuntimeError(lib.lutgemm_strerror(rc).decode())
 
+    def _fused_gemv(self, lins, x, outs, sp, norm=None, gate=None, overwrite=False):
+        """One launch: outs[i] (+)= lins[i](t(x)), t = RMSNorm with weight `norm`, or
+        silu(gate) * x, or identity."""
+        lib, B = native.cabi(), x.shape[0]
+        arr = (native.FusedProblem * len(lins))()
+        for i, (l, o) in enumerate(zip(lins, outs)):
+            arr[i] = native.FusedProblem(l.binaryWeight.data_ptr(), l.alpha.data_ptr(), x.data_ptr(), o.data_ptr(),
+                                         l.N, l.K, l.wbit, l.num_groups, B, int(overwrite),
+                                         norm.data_ptr() if norm is not None else None,
+                                         gate.data_ptr() if gate is not None else None, self.cfg.rms_eps)
+        rc = lib.lutgemm_gemv_rowwise_f16_fused(len(lins), arr, sp)
+        if rc:
+            raise RuntimeError(lib.lutgemm_strerror(rc).decode())
+
     def _step_hip(self):
         cfg, B = self.cfg, self.batch
         hd, H, KV, I = cfg.head_dim, cfg.heads, cfg.kv_heads, cfg.intermediate
@@ -204,23 +219,46 @@ class LutDecoder(nn.Module):
 
         nq, nkv = B * H * hd, B * KV * hd
         q, k, v = self.qkv[:nq], self.qkv[nq:nq + nkv], self.qkv[nq + nkv:]
-        g, u = self.gate_up[:B * I], self.gate_up[B * I:]
+        g, u = self.gate_up[:B * I].view(B, I), self.gate_up[B * I:].view(B, I)
         x, h = self.x_res, self.h_norm
+        # With one or two rows the element-wise work rides inside the look-up kernel
+        # (five launches per block); larger batches go through the matrix-core kernel,
+        # which has no fused transforms, with the glue kernels in between (eight).
+        fold = self.fuse and B <= 2
         torch.index_select(self.embed, 0, self.ids, out=x)
         for li, blk in enumerate(self.blocks):
-            check(lib.lutgemm_decode_rmsnorm_f16(x.data_ptr(), blk.input_norm.data_ptr(), h.data_ptr(), B, cfg.hidden,
-                                                 cfg.rms_eps, self.qkv.data_ptr(), self.qkv.numel() * 2, sp))
-            self._gemv_into([blk.q_proj, blk.k_proj, blk.v_proj], h, [q, k, v], sp)
+            qkv_lins = [blk.q_proj, blk.k_proj, blk.v_proj]
+            if fold and self.fold_norm:
+                self._fused_gemv(qkv_lins, x, [q, k, v], sp, norm=blk.input_norm, overwrite=True)
+            elif fold:
+                check(lib.lutgemm_decode_rmsnorm_f16(x.data_ptr(), blk.input_norm.data_ptr(), h.data_ptr(), B,
+                                                     cfg.hidden, cfg.rms_eps, None, 0, sp))
+                self._fused_gemv(qkv_lins, h, [q, k, v], sp, overwrite=True)
+            else:
+                check(lib.lutgemm_decode_rmsnorm_f16(x.data_ptr(), blk.input_norm.data_ptr(), h.data_ptr(), B,
+                                                     cfg.hidden, cfg.rms_eps, self.qkv.data_ptr(),
+                                                     self.qkv.numel() * 2, sp))
+                self._gemv_into(qkv_lins, h, [q, k, v], sp)
             check(lib.lutgemm_decode_attention_f16(q.data_ptr(), k.data_ptr(), v.data_ptr(), self.cos.data_ptr(),
                                                    self.sin.data_ptr(), self.k_cache[li].data_ptr(),
                                                    self.v_cache[li].data_ptr(), self.pos.data_ptr(),
                                                    self.att.data_ptr(), B, H, KV, hd, cfg.max_positions, sp))
             self._gemv_into([blk.o_proj], self.att, [x], sp)            # x += o_proj(att)
-            check(lib.lutgemm_decode_rmsnorm_f16(x.data_ptr(), blk.post_norm.data_ptr(), h.data_ptr(), B, cfg.hidden,
-                                                 cfg.rms_eps, self.gate_up.data_ptr(), self.gate_up.numel() * 2, sp))
-            self._gemv_into([blk.gate_proj, blk.up_proj], h, [g, u], sp)
-            check(lib.lutgemm_decode_silu_mul_f16(g.data_ptr(), u.data_ptr(), self.act.data_ptr(), B * I, sp))
-            self._gemv_into([blk.down_proj], self.act, [x], sp)         # x += down_proj(act)
+            if fold:
+                if self.fold_norm:
+                    self._fused_gemv([blk.gate_proj, blk.up_proj], x, [g, u], sp, norm=blk.post_norm, overwrite=True)
+                else:
+                    check(lib.lutgemm_decode_rmsnorm_f16(x.data_ptr(), blk.post_norm.data_ptr(), h.data_ptr(), B,
+                                                         cfg.hidden, cfg.rms_eps, None, 0, sp))
+                    self._fused_gemv([blk.gate_proj, blk.up_proj], h, [g, u], sp, overwrite=True)
+                self._fused_gemv([blk.down_proj], u, [x], sp, gate=g)   # x += down_proj(silu(g) * u)
+            else:
+                check(lib.lutgemm_decode_rmsnorm_f16(x.data_ptr(), blk.post_norm.data_ptr(), h.data_ptr(), B,
+                                                     cfg.hidden, cfg.rms_eps, self.gate_up.data_ptr(),
+                                                     self.gate_up.numel() * 2, sp))
+                self._gemv_into([blk.gate_proj, blk.up_proj], h, [g, u], sp)
+                check(lib.lutgemm_decode_silu_mul_f16(g.data_ptr(), u.data_ptr(), self.act.data_ptr(), B * I, sp))
+                self._gemv_into([blk.down_proj], self.act, [x], sp)     # x += down_proj(act)
         check(lib.lutgemm_decode_rmsnorm_f16(x.data_ptr(), self.final_norm.data_ptr(), h.data_ptr(), B, cfg.hidden,
                                              cfg.rms_eps, None, 0, sp))
         torch.matmul(h, self.lm_head.t(), out=self.logits)

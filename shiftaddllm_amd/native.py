@@ -22,6 +22,7 @@ C_ABI_SYMBOLS = (
     "lutgemm_last_hip_error",
     "lutgemm_gemv_rowwise_f16",
     "lutgemm_gemv_rowwise_f16_grouped",
+    "lutgemm_gemv_rowwise_f16_fused",
     "lutgemm_gemv_uniform_f16",
     "lutgemm_gemv_block_f16",
     "lutgemm_gemv_block_shift_u16",
@@ -43,6 +44,15 @@ class RowwiseProblem(ctypes.Structure):
     _fields_ = [("bW", ctypes.c_void_p), ("alpha_f16", ctypes.c_void_p), ("x_f16", ctypes.c_void_p),
                 ("out_f16", ctypes.c_void_p), ("N", ctypes.c_int), ("K", ctypes.c_int),
                 ("nb", ctypes.c_int), ("num_groups", ctypes.c_int), ("M", ctypes.c_int)]
+
+
+class FusedProblem(ctypes.Structure):
+    """struct lutgemm_fused_problem of include/lutgemm_gfx950.h."""
+    _fields_ = [("bW", ctypes.c_void_p), ("alpha_f16", ctypes.c_void_p), ("x_f16", ctypes.c_void_p),
+                ("out_f16", ctypes.c_void_p), ("N", ctypes.c_int), ("K", ctypes.c_int),
+                ("nb", ctypes.c_int), ("num_groups", ctypes.c_int), ("M", ctypes.c_int),
+                ("overwrite", ctypes.c_int), ("norm_weight_f16", ctypes.c_void_p),
+                ("gate_f16", ctypes.c_void_p), ("norm_eps", ctypes.c_float)]
 
 
 class NativeLibraryMissing(ImportError):
@@ -88,6 +98,8 @@ def cabi() -> ctypes.CDLL:
         lib.lutgemm_gemv_rowwise_f16.argtypes = [vp, vp, vp, vp, ci, ci, ci, ci, ci, vp]
         lib.lutgemm_gemv_rowwise_f16_grouped.argtypes = [ci, ctypes.POINTER(RowwiseProblem), vp]
         lib.lutgemm_gemv_rowwise_f16_grouped.restype = ci
+        lib.lutgemm_gemv_rowwise_f16_fused.argtypes = [ci, ctypes.POINTER(FusedProblem), vp]
+        lib.lutgemm_gemv_rowwise_f16_fused.restype = ci
         lib.lutgemm_gemv_uniform_f16.argtypes = [vp, vp, vp, vp, vp, ci, ci, ci, ci, ci, vp]
         lib.lutgemm_gemv_block_f16.argtypes = [vp, vp, vp, vp, ci, ci, ci, ci, ci, vp]
         lib.lutgemm_gemv_block_shift_u16.argtypes = [vp, vp, vp, vp, ci, ci, ci, ci, ci, ci, vp]

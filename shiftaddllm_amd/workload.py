@@ -6,11 +6,9 @@ ShiftAddLLM produces the operands the LUT-GEMM kernels consume:
   * `bcq_shift_quantize`  -- binary-coding quantisation with power-of-two
     scales: greedy initialisation plus alternating refinement, the algorithm of
     quantizers/bcq_quant/bcq_shift.py:82-245 in the ShiftAddLLM checkout
-    (`quantize_shift`, apot_nums = 1).  The least-squares step is solved
-    directly instead of by the reference's fixed-iteration conjugate gradient
-    and the sign assignment is an exhaustive nearest-codeword search instead of
-    the binary search tree; both reach the same optimum of each sub-problem,
-    the emitted bits are not claimed to be identical to the reference's.
+    (`quantize_shift`, apot_nums = 1), restated operation for operation so that
+    it emits the reference's bits (checked against a committed fixture of the
+    reference's own output, tests/golden/bcq_shift_reference.npz).
   * `assign_signs`        -- signs for given scales, quantizers/bcq_quant/quantizer.py:9-37.
   * row-wise problems (groups along K) and "Lat." block problems (8 input
     columns x N/R rows share one scale per bit plane,
@@ -18,6 +16,7 @@ ShiftAddLLM produces the operands the LUT-GEMM kernels consume:
 """
 from __future__ import annotations
 
+import math
 import random
 from dataclasses import dataclass
 
@@ -27,39 +26,69 @@ from .lut_gemm.kernel import pack_binaryWeight
 
 
 def pow2_round(a: torch.Tensor) -> torch.Tensor:
-    """sign(a) * 2^round(log2|a|) (bcq_shift.py:15-39); zero stays zero."""
+    """sign(a) * 2^round(ln|a| / ln 2) (bcq_shift.py:15-39: natural log divided by
+    np.log(2), round-half-to-even); zero stays zero."""
     mag = a.abs()
-    e = torch.round(torch.log2(torch.where(mag > 0, mag, torch.ones_like(mag))))
-    return torch.where(mag > 0, torch.sign(a) * torch.exp2(e), torch.zeros_like(a))
+    e = torch.round(torch.log(torch.where(mag > 0, mag, torch.ones_like(mag))) / math.log(2.0))
+    return torch.where(mag > 0, torch.sign(a) * (2.0 ** e), torch.zeros_like(a))
 
 
 def _codebook(nb: int, device, dtype) -> torch.Tensor:
-    """[2^nb, nb] of +-1, row c has +1 at bit position b iff bit b of c is set."""
+    """[2^nb, nb] of +-1 in the reference's enumeration order (list_binary_vecs,
+    bcq_shift.py:194-198): plane 0 varies slowest, +1 before -1."""
     c = torch.arange(2 ** nb, device=device)
-    bits = (c.unsqueeze(1) >> torch.arange(nb, device=device)) & 1
-    return (bits * 2 - 1).to(dtype)
+    bits = (c.unsqueeze(1) >> torch.arange(nb - 1, -1, -1, device=device)) & 1
+    return (1 - 2 * bits).to(dtype)
 
 
-def assign_signs(w: torch.Tensor, alpha: torch.Tensor, chunk: int = 1 << 22) -> torch.Tensor:
-    """Nearest codeword: w [rows, gs], alpha [rows, nb] -> B [rows, gs, nb] of
-    +-1 minimising |w - sum_b alpha_b B_b| element-wise (the optimum the
-    reference's binary search tree finds, bcq_shift.py:200-224)."""
+def assign_signs(w: torch.Tensor, alpha: torch.Tensor, chunk_rows: int = 1 << 15) -> torch.Tensor:
+    """Nearest codeword: w [rows, gs], alpha [rows, nb] -> B int8 [rows, gs, nb] of +-1
+    minimising |w - sum_b alpha_b B_b| element-wise.  Same result as the reference's
+    binary search tree (find_B_torch, bcq_shift.py:200-224): the 2^nb code values of
+    a row are sorted, a weight goes to the interval of the midpoints it falls in (a
+    weight exactly on a midpoint goes up), equal code values keep the sort's order."""
     rows, gs = w.shape
     nb = alpha.shape[1]
-    book = _codebook(nb, w.device, w.dtype)                  # [C, nb]
-    values = alpha @ book.t()                                # [rows, C]
+    book = _codebook(nb, w.device, torch.float32)            # [C, nb]
     out = torch.empty((rows, gs, nb), dtype=torch.int8, device=w.device)
-    step = max(1, chunk // max(1, gs * (2 ** nb)))
-    for r0 in range(0, rows, step):
-        r1 = min(rows, r0 + step)
-        d = (w[r0:r1].unsqueeze(-1) - values[r0:r1].unsqueeze(1)).abs()   # [r, gs, C]
-        out[r0:r1] = book[d.argmin(dim=-1)].to(torch.int8)
+    book8 = book.to(torch.int8)
+    for r0 in range(0, rows, chunk_rows):
+        r1 = min(rows, r0 + chunk_rows)
+        values = alpha[r0:r1].float().mm(book.t())           # [r, C]
+        vs, order = torch.sort(values)
+        mids = (vs[:, :-1] + vs[:, 1:]) / 2                  # non-decreasing
+        slot = torch.searchsorted(mids, w[r0:r1].float().contiguous(), right=True)   # mids <= w
+        out[r0:r1] = book8[torch.gather(order, 1, slot)]
     return out
+
+
+def _least_squares_cg(gram: torch.Tensor, rhs: torch.Tensor, start: torch.Tensor) -> torch.Tensor:
+    """nb steps of batched conjugate gradient on gram x = rhs from `start`, with the
+    reference's 1e-6 guards in both quotients (batch_cg_torch, bcq_shift.py:226-245).
+    gram [rows, nb, nb], rhs [rows, nb], start [rows, nb]."""
+    rows, nb, _ = gram.shape
+    x = start.clone().view(rows, nb, 1)
+    res = rhs.view(rows, nb, 1) - gram.bmm(x)
+    rr_new = res.transpose(1, 2).bmm(res)
+    direction = res.clone()
+    for _ in range(nb):
+        rr = rr_new
+        gd = gram.bmm(direction)
+        step = rr / (direction.transpose(1, 2).bmm(gd) + 1e-6)
+        x += step * direction
+        res -= step * gd
+        rr_new = res.transpose(1, 2).bmm(res)
+        direction = res + (rr_new / (rr + 1e-6)) * direction
+    return x.view(rows, nb)
 
 
 def bcq_shift_quantize(w: torch.Tensor, nb: int, rounds: int = 5):
     """w [rows, gs] fp32 -> (B int8 [rows, gs, nb], alpha fp32 [rows, nb]) with
-    alpha >= 0, sorted descending, each a power of two after refinement."""
+    alpha >= 0, sorted descending, each a power of two after refinement.
+
+    The reference's quantize_shift(use_bst=True, apot_nums=1) with unit weighting
+    (bcq_shift.py:82-192), float operation for float operation: on the committed
+    fixture of the reference's own output it reproduces B and alpha exactly."""
     w = w.float()
     rows, gs = w.shape
     # greedy: peel off sign * mean|residual| (bcq_shift.py:131-161)
@@ -67,22 +96,23 @@ def bcq_shift_quantize(w: torch.Tensor, nb: int, rounds: int = 5):
     alpha = torch.empty((rows, nb), dtype=torch.float32, device=w.device)
     r = w.clone()
     for b in range(nb):
+        # (the reference takes sign(r), which is 0 for an exact zero; +1 here, so
+        # that every entry packs into one bit)
         s = torch.where(r >= 0, torch.ones_like(r), -torch.ones_like(r))
-        a = r.abs().mean(dim=1)
+        a = r.abs().sum(dim=1) / float(gs)
+        a[torch.isnan(a)] = 0.0
         B[:, :, b] = s
         alpha[:, b] = a
-        r = r - s * a.unsqueeze(1)
+        r -= s * a.view(rows, 1)
     if rounds > 0 and nb > 1:
-        eye = torch.eye(nb, device=w.device).unsqueeze(0)
         for _ in range(rounds):
-            # least squares for alpha given B (bcq_shift.py:163-177,226-245)
-            gram = B.transpose(1, 2) @ B                       # [rows, nb, nb]
-            rhs = B.transpose(1, 2) @ w.unsqueeze(-1)          # [rows, nb, 1]
-            sol = torch.linalg.solve(gram + 1e-4 * eye, rhs).squeeze(-1)
+            # alpha given B: least squares by conjugate gradient from the current alpha,
+            # magnitudes sorted, rounded to powers of two (bcq_shift.py:163-177)
+            Bt = B.transpose(1, 2)
+            sol = _least_squares_cg(Bt.bmm(B), Bt.bmm(w.unsqueeze(-1)).view(rows, nb), alpha)
             alpha = pow2_round(sol.abs().sort(dim=1, descending=True).values)
+            # B given alpha (bcq_shift.py:187-189)
             B = assign_signs(w, alpha).float()
-    else:
-        alpha = alpha
     return B.to(torch.int8), alpha
 
 

@@ -85,3 +85,24 @@ def test_kernels_match_fixtures(fx, gpu_device):
     assert lib.lutgemm_gemv_uniform_f16(p(bW), p(al), p(q), p(x), p(out), 64, 256, 3, 4, 1, sp) == 0
     torch.cuda.synchronize()
     close(out, fx["uni_out"])
+
+
+def test_bcq_quantiser_reproduces_reference_output():
+    """workload.bcq_shift_quantize against (B, alpha) written by the reference's own
+    quantize_shift body (greedy + 5 refinement rounds, BST assignment, one power-of-two
+    term) -- tests/golden/make_bcq_fixture.py made the file from the reference checkout."""
+    import os
+    import numpy as np
+    import torch
+    from shiftaddllm_amd import workload
+    d = np.load(os.path.join(os.path.dirname(__file__), "golden", "bcq_shift_reference.npz"))
+    assert int(d["cases"]) == 4
+    for c in range(int(d["cases"])):
+        w, nb = torch.from_numpy(d[f"w{c}"]), int(d[f"nb{c}"])
+        B, alpha = workload.bcq_shift_quantize(w, nb, rounds=5)
+        assert np.array_equal(alpha.numpy(), d[f"alpha{c}"]), c
+        assert np.array_equal(B.numpy(), d[f"B{c}"]), c
+        # what the fixture itself must satisfy: +-1 signs, descending power-of-two scales
+        assert set(np.unique(d[f"B{c}"])) <= {-1, 1}
+        e = np.log2(d[f"alpha{c}"])
+        assert np.array_equal(e, np.round(e)) and np.all(np.diff(d[f"alpha{c}"], axis=1) <= 0)

@@ -121,3 +121,88 @@ def test_silu_mul(gpu_device, count):
     want = torch.nn.functional.silu(gate.float()).half().float() * up.float()
     assert torch.allclose(out.float(), want, rtol=2e-3, atol=1e-3)
     assert lib.lutgemm_decode_silu_mul_f16(gate.data_ptr(), up.data_ptr(), out.data_ptr(), count + 1, _sp()) == -1
+
+
+# ---- element-wise work folded into the row-wise GEMV ------------------------------------
+
+def _fused_call(lib, lins, x, outs, norm=None, gate=None, overwrite=False, eps=1e-5):
+    arr = (native.FusedProblem * len(lins))()
+    for i, ((bW, alpha, N, K, nb), o) in enumerate(zip(lins, outs)):
+        arr[i] = native.FusedProblem(bW.data_ptr(), alpha.data_ptr(), x.data_ptr(), o.data_ptr(), N, K, nb, K // 128,
+                                     x.shape[0], int(overwrite), norm.data_ptr() if norm is not None else None,
+                                     gate.data_ptr() if gate is not None else None, eps)
+    return lib.lutgemm_gemv_rowwise_f16_fused(len(lins), arr, _sp())
+
+
+def _random_lin(gpu_device, N, K, nb, seed):
+    g = torch.Generator(device=gpu_device).manual_seed(seed)
+    bW = torch.randint(-2 ** 31, 2 ** 31 - 1, (K // 32, nb, N), generator=g, device=gpu_device, dtype=torch.int32)
+    e = torch.randint(-8, -5, (K // 128, 1, N), generator=g, device=gpu_device).float()
+    alpha = torch.exp2(e - torch.arange(nb, device=gpu_device).float().view(1, nb, 1)).half().contiguous()
+    return bW, alpha, N, K, nb
+
+
+def _plain(lib, lin, x, out):
+    bW, alpha, N, K, nb = lin
+    _ok(lib.lutgemm_gemv_rowwise_f16(bW.data_ptr(), alpha.data_ptr(), x.data_ptr(), out.data_ptr(), N, K, nb,
+                                     K // 128, x.shape[0], _sp()))
+
+
+@pytest.mark.parametrize("M,K,Ns,nbs", [(1, 4096, (4096, 1024, 1024), (3, 2, 4)), (2, 1024, (512, 2752), (3, 3)),
+                                          (5, 512, (256,), (2,))])
+def test_fused_rmsnorm_gemv_equals_separate_kernels(gpu_device, M, K, Ns, nbs):
+    """norm folded into the GEMV == rmsnorm kernel followed by the plain GEMV, and both
+    agree with the oracle on the normalised input."""
+    import numpy as np
+    import oracle as orc
+    lib = native.cabi()
+    g = torch.Generator(device=gpu_device).manual_seed(M * 7 + K)
+    x = (torch.randn((M, K), generator=g, device=gpu_device) * 2.5).half()
+    w = (1 + 0.2 * torch.randn((K,), generator=g, device=gpu_device)).half()
+    lins = [_random_lin(gpu_device, N, K, nb, 11 * i + N) for i, (N, nb) in enumerate(zip(Ns, nbs))]
+    h = torch.empty_like(x)
+    _ok(lib.lutgemm_decode_rmsnorm_f16(x.data_ptr(), w.data_ptr(), h.data_ptr(), M, K, 1e-5, None, 0, _sp()))
+    want = [torch.zeros((M, N), dtype=torch.float16, device=gpu_device) for N in Ns]
+    for lin, o in zip(lins, want):
+        _plain(lib, lin, h, o)
+    got = [torch.full((M, N), 9.0, dtype=torch.float16, device=gpu_device) for N in Ns]     # overwritten
+    _ok(_fused_call(lib, lins, x, got, norm=w, overwrite=True))
+    torch.cuda.synchronize()
+    for lin, a, b in zip(lins, got, want):
+        assert torch.allclose(a.float(), b.float(), rtol=2e-3, atol=2e-3 * float(b.float().abs().max()))
+        ref, _ = orc.gemv_rowwise_c(lin[0].cpu().numpy(), lin[1].cpu().numpy(), h.cpu().numpy(), K // 128)
+        rel, mad = orc.error_metrics(a.float().cpu().numpy(), ref.astype(np.float32))
+        assert rel <= 2e-3 and mad <= 1e-2, (rel, mad)
+
+
+@pytest.mark.parametrize("M,K,N,nb", [(1, 11008, 4096, 3), (2, 1408, 512, 4), (4, 512, 256, 2)])
+def test_fused_swiglu_gemv_equals_separate_kernels(gpu_device, M, K, N, nb):
+    lib = native.cabi()
+    g = torch.Generator(device=gpu_device).manual_seed(M * 13 + K)
+    gate = (torch.randn((M, K), generator=g, device=gpu_device) * 2).half()
+    up = torch.randn((M, K), generator=g, device=gpu_device).half()
+    res = torch.randn((M, N), generator=g, device=gpu_device).half()
+    lin = _random_lin(gpu_device, N, K, nb, 5)
+    act = torch.empty_like(up)
+    _ok(lib.lutgemm_decode_silu_mul_f16(gate.data_ptr(), up.data_ptr(), act.data_ptr(), M * K, _sp()))
+    want = res.clone()
+    _plain(lib, lin, act, want)
+    got = res.clone()
+    _ok(_fused_call(lib, [lin], up, [got], gate=gate))                 # accumulates into the residual
+    torch.cuda.synchronize()
+    if M <= 2:
+        assert torch.equal(got, want)                                  # same inputs, same plan: same bits
+    else:                                                              # the plain call took the matrix-core kernel
+        assert torch.allclose(got.float(), want.float(), rtol=2e-3, atol=2e-3 * float(want.float().abs().max()))
+
+
+def test_fused_entry_point_rejects_bad_problems(gpu_device):
+    lib = native.cabi()
+    lin = _random_lin(gpu_device, 256, 512, 2, 1)
+    x = torch.zeros((1, 512), dtype=torch.float16, device=gpu_device)
+    o = torch.zeros((1, 256), dtype=torch.float16, device=gpu_device)
+    assert _fused_call(lib, [lin], x, [o], norm=x, gate=x) == -1       # both transforms
+    assert _fused_call(lib, [lin], x, [o], norm=x, eps=-1.0) == -1
+    arr = (native.FusedProblem * 1)()
+    assert lib.lutgemm_gemv_rowwise_f16_fused(0, arr, _sp()) == -1
+    assert lib.lutgemm_gemv_rowwise_f16_fused(native.MAX_GROUP + 1, arr, _sp()) == -1
