@@ -246,13 +246,24 @@ attention_hd_kernel(const __half *__restrict__ q, const __half *__restrict__ k, 
             v_cache[(cache_row0 + pos) * HD + i] = vv;
         }
     }
-    // key rows of earlier positions do not depend on the above: fetch before the barrier
+    // key and value rows of earlier positions do not depend on the above: fetch them
+    // before the barrier, so that the whole step costs one memory round trip
     const bool first_pass_cached = tid < pos;
     u32x4 row[kChunks];
     if (first_pass_cached) {
         const u32x4 *src = (const u32x4 *)(k_cache + (cache_row0 + tid) * HD);
 #pragma unroll
         for (int c = 0; c < kChunks; ++c) row[c] = src[c];
+    }
+    constexpr int kValueRows = 16;  // value chunks per thread held in registers: 16 * kPosGroups positions
+    const int jg = tid / kChunks, ch = tid % kChunks;
+    const u32x4 *vbase = (const u32x4 *)(v_cache + cache_row0 * HD) + ch;
+    u32x4 vrow[kValueRows];
+#pragma unroll
+    for (int u = 0; u < kValueRows; ++u) {
+        const int j = jg + u * kPosGroups;
+        vrow[u] = (u32x4){0u, 0u, 0u, 0u};
+        if (j < pos) vrow[u] = vbase[(size_t)j * kChunks];
     }
     __syncthreads();
 
@@ -290,26 +301,19 @@ attention_hd_kernel(const __half *__restrict__ q, const __half *__restrict__ k, 
     }
     const float inv = 1.0f / block_reduce<false>(local_sum, red);  // its barriers also publish score[]
 
-    const int jg = tid / kChunks, ch = tid % kChunks;
     float acc[8];
 #pragma unroll
     for (int i = 0; i < 8; ++i) acc[i] = 0.0f;
-    const u32x4 *vbase = (const u32x4 *)(v_cache + cache_row0 * HD) + ch;
-    int j = jg;
-    for (; j + 3 * kPosGroups < pos; j += 4 * kPosGroups) {
-        u32x4 r4[4];
 #pragma unroll
-        for (int u = 0; u < 4; ++u) r4[u] = vbase[(size_t)(j + u * kPosGroups) * kChunks];
+    for (int u = 0; u < kValueRows; ++u) {
+        const int j = jg + u * kPosGroups;
+        float f[8];
+        unpack8(vrow[u], f);
+        const float pj = j < pos ? score[j] : 0.0f;
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
-            float f[8];
-            unpack8(r4[u], f);
-            const float pj = score[j + u * kPosGroups];
-#pragma unroll
-            for (int i = 0; i < 8; ++i) acc[i] = fmaf(pj, f[i], acc[i]);
-        }
+        for (int i = 0; i < 8; ++i) acc[i] = fmaf(pj, f[i], acc[i]);
     }
-    for (; j < pos; j += kPosGroups) {
+    for (int j = jg + kValueRows * kPosGroups; j < pos; j += kPosGroups) {  // longer contexts
         float f[8];
         unpack8(vbase[(size_t)j * kChunks], f);
         const float pj = score[j];
