@@ -854,12 +854,12 @@ __device__ __forceinline__ f16x8 expand_signs(uint32_t w, int beta)
     return __builtin_bit_cast(f16x8, r);
 }
 
+// xs: activations of one round, [wave's step][row][word][instance][8 halves],
+// kMfmaWaves * 16 * MT * kXRowBytes bytes; reused for the final reduction.
 template <int NB, int MT>
-__global__ void __launch_bounds__(kMfmaThreads) lut_gemm_mfma_kernel(const Problem p)
+__device__ __forceinline__ void mfma_tile(const Problem &p, int local_block, char *xs)
 {
-    // activations of one round: [wave's step][row][word][instance][8 halves]; reused for the final reduction
     constexpr int kWaveXBytes = 16 * MT * kXRowBytes;
-    __shared__ __attribute__((aligned(16))) char xs[kMfmaWaves * kWaveXBytes];
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -867,7 +867,7 @@ __global__ void __launch_bounds__(kMfmaThreads) lut_gemm_mfma_kernel(const Probl
     const int li = lane & 15;
     const int kb = lane >> 4;
     int tile, kslice, mchunk;
-    decode_block(p, (int)blockIdx.x, tile, kslice, mchunk);
+    decode_block(p, local_block, tile, kslice, mchunk);
     const int m0 = mchunk * 16 * MT;
     const int n_base = tile * kMfmaTileCols;
 
@@ -953,42 +953,88 @@ __global__ void __launch_bounds__(kMfmaThreads) lut_gemm_mfma_kernel(const Probl
     }
 
     // ---- the 8 waves' accumulators meet in LDS -----------------------------------
+    // red[wave][j = (e*MT + mt)*4 + r][lane], rows padded to 65 words so that the
+    // read-out below (consecutive threads = consecutive outputs) spreads over the banks
+    constexpr int kRedRow = 65;
     __syncthreads();
-    float *red = (float *)xs;  // [wave][e*MT*4 + mt*4 + r][lane]
+    float *red = (float *)xs;
 #pragma unroll
     for (int e = 0; e < 4; ++e)
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
             for (int r = 0; r < 4; ++r)
-                red[(wave * (16 * MT) + (e * MT + mt) * 4 + r) * 64 + lane] = acc[e][mt][r];
+                red[(wave * (16 * MT) + (e * MT + mt) * 4 + r) * kRedRow + lane] = acc[e][mt][r];
     __syncthreads();
-    // thread (wave, lane) finishes values j = wave, wave + 8, ... of lane `lane`
-    for (int j = wave; j < 16 * MT; j += kMfmaWaves) {
+    // Thread t finishes output column t & 63 of rows (t >> 6) + 8*i: a wave covers 64
+    // consecutive outputs of one row, so its atomics and its fp16 read-modify-write
+    // fall into whole cache lines.
+    const int nl = tid & 63;
+    const int n = n_base + nl;
+    const int src_lane = (nl >> 4) * 16;            // kb of the column; + li of the row below
+    const int src_j = (nl & 3) * MT * 4 + ((nl >> 2) & 3);  // e and r of the column; + mt*4 of the row
+    float val[2 * MT];
+    unsigned long long contrib[2 * MT], old[2 * MT];
+#pragma unroll
+    for (int i = 0; i < 2 * MT; ++i) {
+        const int ml = (tid >> 6) + 8 * i;          // row within the chunk
+        const int j = src_j + (ml >> 4) * 4, sl = src_lane + (ml & 15);
         float v = 0.0f;
 #pragma unroll
-        for (int w = 0; w < kMfmaWaves; ++w) v += red[(w * (16 * MT) + j) * 64 + lane];
-        const int e = j / (4 * MT), mt = (j / 4) % MT, r = j & 3;
-        const int m = m0 + 16 * mt + li;
-        const int n = n_base + 16 * kb + 4 * r + e;
+        for (int w = 0; w < kMfmaWaves; ++w) v += red[(w * (16 * MT) + j) * kRedRow + sl];
+        val[i] = v;
+        old[i] = 0;
+        contrib[i] = 0;
+        const int m = m0 + ml;
+        if (p.ksplit > 1 && m < p.M && n < p.N) {
+            v = (v == v) ? v : 65536.0f;
+            v = fminf(fmaxf(v, -65536.0f), 65536.0f);
+            const long long fx = __double2ll_rn((double)v * 4294967296.0);
+            contrib[i] = (unsigned long long)(fx + kBias) + kCountOne;
+            old[i] = __hip_atomic_fetch_add(p.accum + (size_t)m * p.N + n, contrib[i], __ATOMIC_RELAXED,
+                                            __HIP_MEMORY_SCOPE_AGENT);
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < 2 * MT; ++i) {
+        const int m = m0 + (tid >> 6) + 8 * i;
         if (m >= p.M || n >= p.N) continue;
-        __half *out = p.out + (size_t)m * p.N;
+        __half *dst = p.out + (size_t)m * p.N + n;
         if (p.ksplit == 1) {
-            out[n] = __float2half_rn(__half2float(out[n]) + v);
+            *dst = __float2half_rn(__half2float(*dst) + val[i]);
             continue;
         }
-        unsigned long long *accum = p.accum + (size_t)m * p.N;
-        v = (v == v) ? v : 65536.0f;
-        v = fminf(fmaxf(v, -65536.0f), 65536.0f);
-        const long long fx = __double2ll_rn((double)v * 4294967296.0);
-        const unsigned long long contrib = (unsigned long long)(fx + kBias) + kCountOne;
-        const unsigned long long old =
-            __hip_atomic_fetch_add(accum + n, contrib, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        if ((int)(old >> 56) != p.ksplit - 1) continue;
-        const long long total = (long long)((old + contrib) & kSumMask) - (long long)p.ksplit * kBias;
+        if ((int)(old[i] >> 56) != p.ksplit - 1) continue;
+        const long long total = (long long)((old[i] + contrib[i]) & kSumMask) - (long long)p.ksplit * kBias;
         const float y = (float)((double)total * (1.0 / 4294967296.0));
-        out[n] = __float2half_rn(__half2float(out[n]) + y);
-        __hip_atomic_store(accum + n, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        *dst = __float2half_rn(__half2float(*dst) + y);
+        __hip_atomic_store(p.accum + (size_t)m * p.N + n, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+}
+
+template <int NB, int MT>
+__global__ void __launch_bounds__(kMfmaThreads) lut_gemm_mfma_kernel(const Problem p)
+{
+    __shared__ __attribute__((aligned(16))) char xs[kMfmaWaves * 16 * MT * kXRowBytes];
+    mfma_tile<NB, MT>(p, (int)blockIdx.x, xs);
+}
+
+// Several problems in one launch (flat 1-D grid); bit widths may differ.
+template <int MT>
+__global__ void __launch_bounds__(kMfmaThreads) lut_gemm_mfma_group_kernel(const Group g)
+{
+    __shared__ __attribute__((aligned(16))) char xs[kMfmaWaves * 16 * MT * kXRowBytes];
+    const int b = blockIdx.x;
+    int pi = 0;
+#pragma unroll
+    for (int i = 1; i < kMaxGroup; ++i)
+        if (i < g.count && b >= g.p[i].block_begin) pi = i;
+    const Problem &p = g.p[pi];
+    switch (p.nb) {
+    case 1: mfma_tile<1, MT>(p, b - p.block_begin, xs); break;
+    case 2: mfma_tile<2, MT>(p, b - p.block_begin, xs); break;
+    case 3: mfma_tile<3, MT>(p, b - p.block_begin, xs); break;
+    default: mfma_tile<4, MT>(p, b - p.block_begin, xs); break;
     }
 }
 
@@ -1185,8 +1231,12 @@ int mfma_min_rows()
 // 16-output alpha runs.
 bool mfma_eligible(const Problem &p, int mode)
 {
-    return mode == kRowF16 && p.M >= mfma_min_rows() && p.K % kMfmaStepK == 0 && p.group_words % 4 == 0 &&
-           p.N % 16 == 0 && p.N >= 16;
+    if (!(mode == kRowF16 && p.K % kMfmaStepK == 0 && p.group_words % 4 == 0 && p.N % 16 == 0 && p.N >= 16))
+        return false;
+    if (p.M >= mfma_min_rows()) return true;
+    // two rows: the look-up kernel wins only where the sign stream is long enough to
+    // hide its per-row work (measured: 4096x4096x3 13.4 us vs 7.7; 28672x8192x4 51 vs 62)
+    return p.M == 2 && mfma_min_rows() == 3 && (long)p.N * (p.K / 8) * p.nb <= (64l << 20);
 }
 
 template <int NB>
@@ -1202,15 +1252,14 @@ int launch_mfma_nb(const Problem &p, int mt, hipStream_t stream)
     return LUTGEMM_OK;
 }
 
-int run_mfma(Problem &p, hipStream_t stream)
+// K-steps are split 8 ways inside a workgroup already; across workgroups only as
+// far as needed to reach `want_blocks`.
+void plan_mfma(Problem &p, int mt, long want_blocks)
 {
-    const int mt = p.M > 16 ? 2 : 1;
     p.n_tiles = (p.N + kMfmaTileCols - 1) / kMfmaTileCols;
     p.mchunks = (p.M + 16 * mt - 1) / (16 * mt);
     p.nsets = p.K / kMfmaStepK;  // K-steps
-    // K is already split 8 ways inside a workgroup; split it across workgroups only
-    // as far as needed to have about one workgroup per CU
-    long want = 256 / ((long)p.n_tiles * p.mchunks);
+    long want = want_blocks / ((long)p.n_tiles * p.mchunks);
     if (want < 1) want = 1;
     if (want > p.nsets / kMfmaWaves) want = p.nsets / kMfmaWaves;
     if (want < 1) want = 1;
@@ -1219,6 +1268,18 @@ int run_mfma(Problem &p, hipStream_t stream)
     p.sets_per_split = (p.sets_per_split + kMfmaWaves - 1) / kMfmaWaves * kMfmaWaves;  // whole rounds
     p.ksplit = (p.nsets + p.sets_per_split - 1) / p.sets_per_split;
     p.n_blocks = p.n_tiles * p.ksplit * p.mchunks;
+}
+
+int mfma_blocks()
+{
+    static const int v = env_int("LUTGEMM_MFMA_BLOCKS", 256);
+    return v;
+}
+
+int run_mfma(Problem &p, hipStream_t stream)
+{
+    const int mt = p.M > 16 ? 2 : 1;
+    plan_mfma(p, mt, mfma_blocks());
     if (p.ksplit > 1) {
         int rc = get_workspace(stream, (size_t)p.M * p.N, &p.accum);
         if (rc != LUTGEMM_OK) return rc;
@@ -1230,6 +1291,47 @@ int run_mfma(Problem &p, hipStream_t stream)
     case 4: return launch_mfma_nb<4>(p, mt, stream);
     default: return LUTGEMM_EINVAL;
     }
+}
+
+// All problems of a group on the matrix-core kernel in one launch (they share the
+// row-tile height: all M <= 16 or all M > 16).
+int run_mfma_group(Group &g, hipStream_t stream)
+{
+    const int mt = g.p[0].M > 16 ? 2 : 1;
+    long total_bytes = 0;
+    size_t words = 0;
+    for (int i = 0; i < g.count; ++i) {
+        total_bytes += (long)g.p[i].N * (g.p[i].K / 8) * g.p[i].nb;
+        words += (size_t)g.p[i].M * g.p[i].N;
+    }
+    int begin = 0;
+    bool any_split = false;
+    for (int i = 0; i < g.count; ++i) {
+        Problem &p = g.p[i];
+        const long mine = (long)p.N * (p.K / 8) * p.nb;
+        plan_mfma(p, mt, (long)mfma_blocks() * mine / (total_bytes > 0 ? total_bytes : 1));
+        p.block_begin = begin;
+        begin += p.n_blocks;
+        any_split = any_split || p.ksplit > 1;
+    }
+    if (any_split) {
+        unsigned long long *base = nullptr;
+        int rc = get_workspace(stream, words, &base);
+        if (rc != LUTGEMM_OK) return rc;
+        size_t off = 0;
+        for (int i = 0; i < g.count; ++i) {
+            g.p[i].accum = base + off;
+            off += (size_t)g.p[i].M * g.p[i].N;
+        }
+    }
+    const dim3 grid((unsigned)begin), block(kMfmaThreads);
+    if (mt == 2)
+        hipLaunchKernelGGL((lut_gemm_mfma_group_kernel<2>), grid, block, 0, stream, g);
+    else
+        hipLaunchKernelGGL((lut_gemm_mfma_group_kernel<1>), grid, block, 0, stream, g);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return hip_fail(e);
+    return LUTGEMM_OK;
 }
 
 int run(int mode, const uint32_t *bW, const void *alpha, const void *qbias, const void *x,
@@ -1300,6 +1402,9 @@ int run_group(int count, const lutgemm_fused_problem *problems, hipStream_t stre
         total_bytes += (long)q.N * (q.K / 8) * q.nb * q.M;
     }
     if (plain && all_mfma) {
+        bool same_height = true;
+        for (int i = 1; i < count; ++i) same_height = same_height && ((g.p[i].M > 16) == (g.p[0].M > 16));
+        if (count > 1 && same_height) return run_mfma_group(g, stream);
         for (int i = 0; i < count; ++i) {
             int rc = run_mfma(g.p[i], stream);
             if (rc != LUTGEMM_OK) return rc;
