@@ -1270,16 +1270,20 @@ void plan_mfma(Problem &p, int mt, long want_blocks)
     p.n_blocks = p.n_tiles * p.ksplit * p.mchunks;
 }
 
-int mfma_blocks()
+// Workgroups wanted per launch: two per CU for the 16-row tile (its register count
+// lets two be resident), one per CU for the 32-row tile.  Measured, 8192x8192x2:
+// 16 rows 16.9 us at 256 and 15.1 at 512; 32 rows 36.4 at 256 and 40.0 at 512 (4 bits).
+int mfma_blocks(int mt)
 {
-    static const int v = env_int("LUTGEMM_MFMA_BLOCKS", 256);
-    return v;
+    static const int v = env_int("LUTGEMM_MFMA_BLOCKS", 0);
+    if (v > 0) return v;
+    return mt == 1 ? 512 : 256;
 }
 
 int run_mfma(Problem &p, hipStream_t stream)
 {
     const int mt = p.M > 16 ? 2 : 1;
-    plan_mfma(p, mt, mfma_blocks());
+    plan_mfma(p, mt, mfma_blocks(mt));
     if (p.ksplit > 1) {
         int rc = get_workspace(stream, (size_t)p.M * p.N, &p.accum);
         if (rc != LUTGEMM_OK) return rc;
@@ -1309,7 +1313,7 @@ int run_mfma_group(Group &g, hipStream_t stream)
     for (int i = 0; i < g.count; ++i) {
         Problem &p = g.p[i];
         const long mine = (long)p.N * (p.K / 8) * p.nb;
-        plan_mfma(p, mt, (long)mfma_blocks() * mine / (total_bytes > 0 ? total_bytes : 1));
+        plan_mfma(p, mt, (long)mfma_blocks(mt) * mine / (total_bytes > 0 ? total_bytes : 1));
         p.block_begin = begin;
         begin += p.n_blocks;
         any_split = any_split || p.ksplit > 1;

@@ -190,7 +190,7 @@ def test_fused_swiglu_gemv_equals_separate_kernels(gpu_device, M, K, N, nb):
     got = res.clone()
     _ok(_fused_call(lib, [lin], up, [got], gate=gate))                 # accumulates into the residual
     torch.cuda.synchronize()
-    if M <= 2:
+    if M == 1:
         assert torch.equal(got, want)                                  # same inputs, same plan: same bits
     else:                                                              # the plain call took the matrix-core kernel
         assert torch.allclose(got.float(), want.float(), rtol=2e-3, atol=2e-3 * float(want.float().abs().max()))
@@ -226,7 +226,10 @@ def test_sum_of_squares_hand_over(gpu_device, M, K, N, nb):
     want_out = res.clone()
     _plain(lib, lin, x, want_out)
     torch.cuda.synchronize()
-    assert torch.equal(out, want_out)
+    if M == 1:
+        assert torch.equal(out, want_out)
+    else:                                                              # the plain call took the matrix-core kernel
+        assert torch.allclose(out.float(), want_out.float(), rtol=2e-3, atol=2e-3 * float(want_out.float().abs().max()))
     o32 = out.float()
     want = ((o32 * o32).clamp(max=1.0e12) * 16777216.0).to(torch.int64).sum(dim=1)     # truncation, as in the kernel
     assert torch.equal(slots.sum(dim=1), want)
