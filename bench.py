@@ -343,9 +343,12 @@ def main():
             torch.cuda.empty_cache()
         decode_res["config"] = ("random-init Llama-2-7B, 32 blocks, per-linear bits drawn 2:3:3:4 by "
                                 f"random.Random(0) ({counts[2]}x2-bit, {counts[3]}x3-bit, {counts[4]}x4-bit), "
-                                "group 128, fp16 RMSNorm/RoPE/attention in torch, 128 prompt tokens fed one by "
-                                "one then 128 greedy tokens, one HIP-graph replay + sync per token, "
-                                "q/k/v and gate/up as fused launches")
+                                "group 128, 128 prompt tokens fed one by one then 128 greedy tokens, one "
+                                "HIP-graph replay + sync per token; q/k/v and gate/up as grouped launches; "
+                                "batch 1: RMSNorm and SiLU*up folded into the look-up GEMVs, rotary + KV append "
+                                "+ attention in one HIP kernel (5 launches per block); batch 8: matrix-core "
+                                "GEMM kernel with RMSNorm / attention / SiLU*up HIP kernels between (8 launches "
+                                "per block); embedding gather and fp16 lm_head in torch")
 
     traffic = None
     if os.path.exists(TRAFFIC_NOTE):
