@@ -35,8 +35,6 @@
 extern "C" {
 #endif
 
-#define LUTGEMM_SUMSQ_SLOTS 16 /* uint64 words per row of a sum-of-squares hand-over */
-
 #define LUTGEMM_OK 0
 #define LUTGEMM_EINVAL (-1)   /* bad shape / size / null pointer            */
 #define LUTGEMM_EALIGN (-2)   /* pointer not aligned as required            */
@@ -163,17 +161,7 @@ int lutgemm_release_workspaces(void);
  *                     fp16(fp16(silu(gate)) * x)  (SwiGLU);
  *                     at most one of the two per problem; both 16-byte aligned;
  *   overwrite       : 0 = out += y like every other entry point, 1 = out = y
- *                     (out need not be initialised);
- *   sumsq_out       : NULL, or uint64 [M][LUTGEMM_SUMSQ_SLOTS], zero before the
- *                     call: the launch adds, spread over the slots of row m, the
- *                     squares of the values it leaves in out[m] (as rounded to
- *                     fp16), in units of 2^-24 -- integer sums, so the total does
- *                     not depend on the order in which outputs complete;
- *   sumsq_in        : NULL, or such an array completed by an EARLIER launch for
- *                     the rows of x; needs norm_weight_f16.  The reciprocal RMS
- *                     is then taken from it instead of being re-formed from x by
- *                     every workgroup (o_proj -> post-attention norm -> gate/up;
- *                     down_proj -> next block's input norm -> q/k/v).
+ *                     (out need not be initialised).
  * A problem with none of the three is the plain row-wise GEMV.  The problems of
  * one call must share their transform (all norm, all gate or all none;
  * LUTGEMM_EUNSUP otherwise).  Problems with a transform or with overwrite run on
@@ -189,8 +177,6 @@ typedef struct lutgemm_fused_problem {
     const void *norm_weight_f16;
     const void *gate_f16;
     float norm_eps;
-    void *sumsq_out;
-    const void *sumsq_in;
 } lutgemm_fused_problem;
 
 int lutgemm_gemv_rowwise_f16_fused(int count, const lutgemm_fused_problem *problems, void *stream);

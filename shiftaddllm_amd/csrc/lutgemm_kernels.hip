@@ -67,7 +67,6 @@ constexpr int kLutDwords = 256 * kEntryStride;  // 64 KiB: two interleaved table
 constexpr int kStageDwords = 2 * 2 * 4 * kTables;  // staged block alphas: [buffer][row group][bit][chunk]
 constexpr int kMaxKSplit = 32;             // bounded by the fixed-point accumulator layout
 constexpr int kMaxGroup = LUTGEMM_MAX_GROUP;  // problems per grouped launch
-constexpr int kSumsqSlots = LUTGEMM_SUMSQ_SLOTS;  // addresses a row's sum of squares is spread over
 
 // fixed-point accumulator word: [63:56] contributions, [55:0] sum of (v + kBias),
 // v = partial * 2^32 with |partial| <= 2^16
@@ -118,11 +117,6 @@ struct Problem {
     const __half *gate;    // non-null [M][K]: the input is fp16(fp16(silu(gate)) * x)
     float norm_eps;
     int overwrite;         // 1: out = y instead of out += y
-    // sums of squares of the rows of `out`, handed from the launch that completes
-    // them to the launch that normalises by them: [M][kSumsqSlots] words in units
-    // of 2^-24, zero before the producing launch
-    unsigned long long *sumsq_out;
-    const unsigned long long *sumsq_in;
 };
 
 // Flat workgroup index (relative to the problem) -> (tile, kslice, m).
@@ -445,7 +439,7 @@ __device__ __forceinline__ void lookup_set(const SetOperands<NB, NSTEPS, MODE> &
 // mchunk*MROWS .. +MROWS-1.  The sign words of a set are loaded once and used
 // for all MROWS rows; tables are built per (set, row) and double buffered, so the
 // work items of the pipeline are the (set, row) pairs in order.
-template <int NB, int NSTEPS, int MODE, int MROWS, int XF = kXNone, bool SQ = false>
+template <int NB, int NSTEPS, int MODE, int MROWS, int XF = kXNone>
 __device__ __forceinline__ void gemv_tile(const Problem &p, int tile, int kslice, int mchunk, float *lut)
 {
     const int tid = threadIdx.x;
@@ -517,7 +511,7 @@ __device__ __forceinline__ void gemv_tile(const Problem &p, int tile, int kslice
     constexpr int kNormChunks = 2;  // 16-byte chunks per thread held in registers: K <= 8192
     u32x4 nx[XF == kXNorm ? MROWS : 1][kNormChunks];
     if constexpr (XF == kXNorm) {
-        if (p.sumsq_in == nullptr) {
+        {
 #pragma unroll
             for (int r = 0; r < MROWS; ++r)
 #pragma unroll
@@ -543,17 +537,7 @@ __device__ __forceinline__ void gemv_tile(const Problem &p, int tile, int kslice
 #pragma unroll
     for (int r = 0; r < MROWS; ++r) rscale[r] = 1.0f;
     if constexpr (XF == kXNorm) {
-        if (p.sumsq_in != nullptr) {
-            // the launch that wrote x left the sum of squares of each row behind
-#pragma unroll
-            for (int r = 0; r < MROWS; ++r) {
-                const unsigned long long *slot = p.sumsq_in + (size_t)min(m0 + r, p.M - 1) * kSumsqSlots;
-                unsigned long long t = 0;
-#pragma unroll
-                for (int i = 0; i < kSumsqSlots; ++i) t += slot[i];
-                rscale[r] = rsqrtf((float)((double)t * (1.0 / 16777216.0)) / (float)p.K + p.norm_eps);
-            }
-        } else {
+        {
             float ss[MROWS];
 #pragma unroll
             for (int r = 0; r < MROWS; ++r) {
@@ -654,17 +638,6 @@ __device__ __forceinline__ void gemv_tile(const Problem &p, int tile, int kslice
             }
     if (kw != 0) return;
 
-    // squares of the values this lane writes, in 2^-24 units: integer sums are the
-    // same whatever the order in which workgroups complete their outputs
-    unsigned long long sq[MROWS];
-#pragma unroll
-    for (int r = 0; r < MROWS; ++r) sq[r] = 0;
-    auto square_fx = [](uint32_t half_bits) -> unsigned long long {
-        const float v = half_bits_to_float(half_bits);
-        const float q = fminf(v * v, 1.0e12f) * 16777216.0f;  // non-finite values saturate
-        return (q == q) ? (unsigned long long)q : 0ull;
-    };
-
 #pragma unroll
     for (int r = 0; r < MROWS; ++r) {
         const int m = m0 + r;
@@ -684,9 +657,6 @@ __device__ __forceinline__ void gemv_tile(const Problem &p, int tile, int kslice
                     raw.x = float_to_half_bits(o0) | (float_to_half_bits(o1) << 16);
                     raw.y = float_to_half_bits(o2) | (float_to_half_bits(o3) << 16);
                     *(u32x2 *)(out + n) = raw;
-                    if constexpr (SQ)
-                        sq[r] += square_fx(raw.x & 0xffffu) + square_fx(raw.x >> 16) + square_fx(raw.y & 0xffffu) +
-                                 square_fx(raw.y >> 16);
                 }
             }
             continue;
@@ -725,26 +695,8 @@ __device__ __forceinline__ void gemv_tile(const Problem &p, int tile, int kslice
                     (long long)((old[s][i] + contrib[s][i]) & kSumMask) - (long long)p.ksplit * kBias;
                 const float y = (float)((double)total * (1.0 / 4294967296.0));
                 const float prev = p.overwrite ? 0.0f : half_bits_to_float((raw2[i >> 1] >> (16 * (i & 1))) & 0xffffu);
-                const uint32_t o_bits = float_to_half_bits(prev + y);
-                out[n + i] = __ushort_as_half((unsigned short)o_bits);
+                out[n + i] = __float2half_rn(prev + y);
                 __hip_atomic_store(accum + n + i, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                if constexpr (SQ) sq[r] += square_fx(o_bits);
-            }
-        }
-    }
-    if constexpr (SQ) {
-        if (p.sumsq_out != nullptr) {
-            // the 8 lanes of a wave still here are 0..3 and 32..35
-#pragma unroll
-            for (int r = 0; r < MROWS; ++r) {
-                unsigned long long t = sq[r];
-                t += __shfl_xor(t, 1);
-                t += __shfl_xor(t, 2);
-                t += __shfl_xor(t, 32);
-                if (lane == 0 && t != 0 && m0 + r < p.M)
-                    __hip_atomic_fetch_add(p.sumsq_out + (size_t)(m0 + r) * kSumsqSlots +
-                                               ((tile * kWaves + wave) & (kSumsqSlots - 1)),
-                                           t, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             }
         }
     }
@@ -776,10 +728,10 @@ lut_gemv_group_kernel(const Group g)
     int tile, kslice, m;
     decode_block(p, b - p.block_begin, tile, kslice, m);
     switch (p.nb) {
-    case 1: gemv_tile<1, NSTEPS, kRowF16, 1, XF, true>(p, tile, kslice, m, lut); break;
-    case 2: gemv_tile<2, NSTEPS, kRowF16, 1, XF, true>(p, tile, kslice, m, lut); break;
-    case 3: gemv_tile<3, NSTEPS, kRowF16, 1, XF, true>(p, tile, kslice, m, lut); break;
-    default: gemv_tile<4, NSTEPS, kRowF16, 1, XF, true>(p, tile, kslice, m, lut); break;
+    case 1: gemv_tile<1, NSTEPS, kRowF16, 1, XF>(p, tile, kslice, m, lut); break;
+    case 2: gemv_tile<2, NSTEPS, kRowF16, 1, XF>(p, tile, kslice, m, lut); break;
+    case 3: gemv_tile<3, NSTEPS, kRowF16, 1, XF>(p, tile, kslice, m, lut); break;
+    default: gemv_tile<4, NSTEPS, kRowF16, 1, XF>(p, tile, kslice, m, lut); break;
     }
 }
 
@@ -1392,15 +1344,11 @@ int run_group(int count, const lutgemm_fused_problem *problems, hipStream_t stre
         p.gate = (const __half *)q.gate_f16;
         p.norm_eps = q.norm_eps;
         p.overwrite = q.overwrite;
-        if (q.sumsq_in && !q.norm_weight_f16) return LUTGEMM_EINVAL;
-        if (!aligned(q.sumsq_out, 8) || !aligned(q.sumsq_in, 8)) return LUTGEMM_EALIGN;
-        p.sumsq_out = (unsigned long long *)q.sumsq_out;
-        p.sumsq_in = (const unsigned long long *)q.sumsq_in;
         // one kernel instance per transform: the problems of a launch share theirs
         const int mine = p.norm_w ? kXNorm : p.gate ? kXGate : kXNone;
         if (i > 0 && mine != xform) return LUTGEMM_EUNSUP;
         xform = mine;
-        plain = plain && !p.norm_w && !p.gate && !p.overwrite && !p.sumsq_out;
+        plain = plain && !p.norm_w && !p.gate && !p.overwrite;
         all_mfma = all_mfma && mfma_eligible(p, kRowF16);
         words += (size_t)q.M * q.N;
         total_bytes += (long)q.N * (q.K / 8) * q.nb * q.M;

@@ -103,7 +103,9 @@ class LutDecoder(nn.Module):
         if glue not in ("hip", "torch"):
             raise ValueError(f"glue must be 'hip' or 'torch', got {glue!r}")
         self.cfg, self.batch, self.fuse, self.glue = cfg, batch, fuse_launches, glue
-        self.fold_norm = True
+        # RMSNorm inside the q,k,v and gate,up GEMVs instead of a kernel of its own: measured equal
+        # (every workgroup re-reads the row to form its RMS), so the separate kernel stays the default
+        self.fold_norm = False
         dev = torch.device(device)
         gen = torch.Generator(device=dev).manual_seed(seed)
         names = ("self_attn.q_proj", "self_attn.k_proj", "self_attn.v_proj", "self_attn.o_proj",
@@ -140,8 +142,6 @@ class LutDecoder(nn.Module):
         self.register_buffer("att", torch.zeros((batch, H), **f16), persistent=False)
         self.register_buffer("gate_up", torch.zeros((2 * batch * I,), **f16), persistent=False)
         self.register_buffer("act", torch.zeros((batch, I), **f16), persistent=False)
-        self.register_buffer("sumsq", torch.zeros((2 * cfg.layers + 1, batch, native.SUMSQ_SLOTS), dtype=torch.int64,
-                                                  device=dev), persistent=False)
         self._graph = None
         self._stream = None
 
@@ -195,19 +195,16 @@ class LutDecoder(nn.Module):
             if rc:
                 raise RuntimeError(lib.lutgemm_strerror(rc).decode())
 
-    def _fused_gemv(self, lins, x, outs, sp, norm=None, gate=None, overwrite=False, sumsq_out=None, sumsq_in=None):
+    def _fused_gemv(self, lins, x, outs, sp, norm=None, gate=None, overwrite=False):
         """One launch: outs[i] (+)= lins[i](t(x)), t = RMSNorm with weight `norm`, or
-        silu(gate) * x, or identity.  sumsq_out: the launch also leaves the sum of
-        squares of each row of its output there; sumsq_in: RMSNorm takes it from there."""
+        silu(gate) * x, or identity."""
         lib, B = native.cabi(), x.shape[0]
         arr = (native.FusedProblem * len(lins))()
         for i, (l, o) in enumerate(zip(lins, outs)):
             arr[i] = native.FusedProblem(l.binaryWeight.data_ptr(), l.alpha.data_ptr(), x.data_ptr(), o.data_ptr(),
                                          l.N, l.K, l.wbit, l.num_groups, B, int(overwrite),
                                          norm.data_ptr() if norm is not None else None,
-                                         gate.data_ptr() if gate is not None else None, self.cfg.rms_eps,
-                                         sumsq_out.data_ptr() if sumsq_out is not None else None,
-                                         sumsq_in.data_ptr() if sumsq_in is not None else None)
+                                         gate.data_ptr() if gate is not None else None, self.cfg.rms_eps)
         rc = lib.lutgemm_gemv_rowwise_f16_fused(len(lins), arr, sp)
         if rc:
             raise RuntimeError(lib.lutgemm_strerror(rc).decode())
@@ -231,16 +228,10 @@ class LutDecoder(nn.Module):
         # which has no fused transforms, with the glue kernels in between (eight).
         fold = self.fuse and B <= 2
         torch.index_select(self.embed, 0, self.ids, out=x)
-        # sums of squares of the residual stream, handed from the GEMV that completes
-        # it to the GEMVs that normalise it: one slot set per norm, cleared per step
-        ssq = self.sumsq if (fold and self.fold_norm) else None
-        if ssq is not None:
-            ssq.zero_()
         for li, blk in enumerate(self.blocks):
             qkv_lins = [blk.q_proj, blk.k_proj, blk.v_proj]
             if fold and self.fold_norm:
-                self._fused_gemv(qkv_lins, x, [q, k, v], sp, norm=blk.input_norm, overwrite=True,
-                                 sumsq_in=ssq[2 * li] if li > 0 else None)
+                self._fused_gemv(qkv_lins, x, [q, k, v], sp, norm=blk.input_norm, overwrite=True)
             elif fold:
                 check(lib.lutgemm_decode_rmsnorm_f16(x.data_ptr(), blk.input_norm.data_ptr(), h.data_ptr(), B,
                                                      cfg.hidden, cfg.rms_eps, None, 0, sp))
@@ -254,20 +245,15 @@ class LutDecoder(nn.Module):
                                                    self.sin.data_ptr(), self.k_cache[li].data_ptr(),
                                                    self.v_cache[li].data_ptr(), self.pos.data_ptr(),
                                                    self.att.data_ptr(), B, H, KV, hd, cfg.max_positions, sp))
-            if ssq is not None:                                          # x += o_proj(att)
-                self._fused_gemv([blk.o_proj], self.att, [x], sp, sumsq_out=ssq[2 * li + 1])
-            else:
-                self._gemv_into([blk.o_proj], self.att, [x], sp)
+            self._gemv_into([blk.o_proj], self.att, [x], sp)            # x += o_proj(att)
             if fold:
                 if self.fold_norm:
-                    self._fused_gemv([blk.gate_proj, blk.up_proj], x, [g, u], sp, norm=blk.post_norm, overwrite=True,
-                                     sumsq_in=ssq[2 * li + 1])
+                    self._fused_gemv([blk.gate_proj, blk.up_proj], x, [g, u], sp, norm=blk.post_norm, overwrite=True)
                 else:
                     check(lib.lutgemm_decode_rmsnorm_f16(x.data_ptr(), blk.post_norm.data_ptr(), h.data_ptr(), B,
                                                          cfg.hidden, cfg.rms_eps, None, 0, sp))
                     self._fused_gemv([blk.gate_proj, blk.up_proj], h, [g, u], sp, overwrite=True)
-                self._fused_gemv([blk.down_proj], u, [x], sp, gate=g,   # x += down_proj(silu(g) * u)
-                                 sumsq_out=ssq[2 * li + 2] if ssq is not None else None)
+                self._fused_gemv([blk.down_proj], u, [x], sp, gate=g)   # x += down_proj(silu(g) * u)
             else:
                 check(lib.lutgemm_decode_rmsnorm_f16(x.data_ptr(), blk.post_norm.data_ptr(), h.data_ptr(), B,
                                                      cfg.hidden, cfg.rms_eps, self.gate_up.data_ptr(),

@@ -37,7 +37,6 @@ C_ABI_SYMBOLS = (
 
 
 MAX_GROUP = 8
-SUMSQ_SLOTS = 16
 
 
 class RowwiseProblem(ctypes.Structure):
@@ -53,8 +52,7 @@ class FusedProblem(ctypes.Structure):
                 ("out_f16", ctypes.c_void_p), ("N", ctypes.c_int), ("K", ctypes.c_int),
                 ("nb", ctypes.c_int), ("num_groups", ctypes.c_int), ("M", ctypes.c_int),
                 ("overwrite", ctypes.c_int), ("norm_weight_f16", ctypes.c_void_p),
-                ("gate_f16", ctypes.c_void_p), ("norm_eps", ctypes.c_float),
-                ("sumsq_out", ctypes.c_void_p), ("sumsq_in", ctypes.c_void_p)]
+                ("gate_f16", ctypes.c_void_p), ("norm_eps", ctypes.c_float)]
 
 
 class NativeLibraryMissing(ImportError):

@@ -206,47 +206,3 @@ def test_fused_entry_point_rejects_bad_problems(gpu_device):
     arr = (native.FusedProblem * 1)()
     assert lib.lutgemm_gemv_rowwise_f16_fused(0, arr, _sp()) == -1
     assert lib.lutgemm_gemv_rowwise_f16_fused(native.MAX_GROUP + 1, arr, _sp()) == -1
-
-
-@pytest.mark.parametrize("M,K,N,nb", [(1, 4096, 4096, 3), (2, 512, 1024, 2), (1, 11008, 4096, 4)])
-def test_sum_of_squares_hand_over(gpu_device, M, K, N, nb):
-    """A launch with sumsq_out leaves exactly the fixed-point sum of the squares of its
-    fp16 outputs; a norm-folding launch fed with it equals one that re-forms the RMS."""
-    lib = native.cabi()
-    g = torch.Generator(device=gpu_device).manual_seed(M + K + N)
-    x = torch.randn((M, K), generator=g, device=gpu_device).half()
-    res = (torch.randn((M, N), generator=g, device=gpu_device) * 3).half()
-    lin = _random_lin(gpu_device, N, K, nb, 3)
-    arr = (native.FusedProblem * 1)()
-    slots = torch.zeros((M, native.SUMSQ_SLOTS), dtype=torch.int64, device=gpu_device)
-    out = res.clone()
-    arr[0] = native.FusedProblem(lin[0].data_ptr(), lin[1].data_ptr(), x.data_ptr(), out.data_ptr(), N, K, nb, K // 128,
-                                 M, 0, None, None, 0.0, slots.data_ptr(), None)
-    _ok(lib.lutgemm_gemv_rowwise_f16_fused(1, arr, _sp()))
-    want_out = res.clone()
-    _plain(lib, lin, x, want_out)
-    torch.cuda.synchronize()
-    if M == 1:
-        assert torch.equal(out, want_out)
-    else:                                                              # the plain call took the matrix-core kernel
-        assert torch.allclose(out.float(), want_out.float(), rtol=2e-3, atol=2e-3 * float(want_out.float().abs().max()))
-    o32 = out.float()
-    want = ((o32 * o32).clamp(max=1.0e12) * 16777216.0).to(torch.int64).sum(dim=1)     # truncation, as in the kernel
-    assert torch.equal(slots.sum(dim=1), want)
-
-    # consumer: the next layer normalises `out` (K2 = N) with the handed-over sums
-    lin2 = _random_lin(gpu_device, 256, N, 3, 9)
-    w = (1 + 0.1 * torch.randn((N,), generator=g, device=gpu_device)).half()
-    a = torch.empty((M, 256), dtype=torch.float16, device=gpu_device)
-    b = torch.empty_like(a)
-    for dst, sumsq in ((a, slots), (b, None)):
-        arr[0] = native.FusedProblem(lin2[0].data_ptr(), lin2[1].data_ptr(), out.data_ptr(), dst.data_ptr(), 256, N, 3,
-                                     N // 128, M, 1, w.data_ptr(), None, 1e-5, None,
-                                     sumsq.data_ptr() if sumsq is not None else None)
-        _ok(lib.lutgemm_gemv_rowwise_f16_fused(1, arr, _sp()))
-    torch.cuda.synchronize()
-    assert torch.allclose(a.float(), b.float(), rtol=2e-3, atol=2e-3 * float(b.float().abs().max()))
-    # sumsq_in without a norm weight is rejected
-    arr[0] = native.FusedProblem(lin2[0].data_ptr(), lin2[1].data_ptr(), out.data_ptr(), a.data_ptr(), 256, N, 3,
-                                 N // 128, M, 1, None, None, 1e-5, None, slots.data_ptr())
-    assert lib.lutgemm_gemv_rowwise_f16_fused(1, arr, _sp()) == -1

@@ -459,8 +459,12 @@ def test_decoder_matches_dense_dequantised_model(gpu_device):
     lut.glue, lut.fuse = "torch", True
     got_torch_glue = run(lut, capture=False)
     lut.glue = "hip"
+    # RMSNorm folded into the q,k,v and gate,up launches (the decoder's default keeps it separate)
+    lut.fold_norm = True
+    got_fold_norm = run(lut, capture=False)
+    lut.fold_norm = False
     for name, got in (("fused", got_fused), ("graph", got_graph), ("plain", got_plain),
-                      ("torch glue", got_torch_glue)):
+                      ("torch glue", got_torch_glue), ("folded norm", got_fold_norm)):
         rel, mad = orc.error_metrics(got.numpy(), want.numpy())
         assert rel <= REL_L2_BAR and mad <= MAX_ABS_BAR, (name, rel, mad)
     # replaying the graph gives what the eager fused path gave
