@@ -51,6 +51,8 @@ def parse_args():
                     help="only the 224-launch step (no fused sequences, no per-shape table): for profiler runs")
     ap.add_argument("--profile-shape", type=str, default="",
                     help="N,K[,nb[,iters[,M]]]: only launch this shape repeatedly (for rocprofv3 runs) and exit")
+    ap.add_argument("--profile-decode", type=int, default=0,
+                    help="batch: only replay ten graph-captured decode steps of the 7B decoder (for rocprofv3 runs) and exit")
     ap.add_argument("--profile-copy", type=int, default=0,
                     help="bytes: only run the calibration copy kernel a few times (for rocprofv3 --pmc) and exit")
     return ap.parse_args()
@@ -116,6 +118,17 @@ def main():
                 lib.lutgemm_copy_bytes(ctypes.c_void_p(dst.data_ptr()), ctypes.c_void_p(src.data_ptr()), nbytes, sp)
         stream.synchronize()
         print(json.dumps({"copy_bytes": nbytes, "launches": 5}))
+        return
+    if args.profile_decode:
+        from shiftaddllm_amd import decode
+        qc = workload.mixed_bit_config(decode.LLAMA2_7B.layers, seed=0)
+        model = decode.LutDecoder(decode.LLAMA2_7B, qc, batch=args.profile_decode, seed=0, device=dev)
+        model.capture()
+        ids = torch.randint(0, decode.LLAMA2_7B.vocab_size, (args.profile_decode,), device=dev)
+        for t in range(100, 110):
+            model.forward_token(ids, t)
+        torch.cuda.synchronize()
+        print(json.dumps({"decode_batch": args.profile_decode, "steps": 10, "positions": [100, 109]}))
         return
     if args.profile_shape:
         parts = [int(v) for v in args.profile_shape.split(",")]
