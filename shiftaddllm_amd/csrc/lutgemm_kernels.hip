@@ -1187,8 +1187,9 @@ bool mfma_eligible(const Problem &p, int mode)
         return false;
     if (p.M >= mfma_min_rows()) return true;
     // two rows: the look-up kernel wins only where the sign stream is long enough to
-    // hide its per-row work (measured: 4096x4096x3 13.4 us vs 7.7; 28672x8192x4 51 vs 62)
-    return p.M == 2 && mfma_min_rows() == 3 && (long)p.N * (p.K / 8) * p.nb <= (64l << 20);
+    // hide its per-row work (measured, look-up vs matrix core: 4096x4096x3 13.4 us vs
+    // 7.4; 8192x8192x4 21.8 vs 19.9; 28672x8192x2 about 30 vs 38.9; 28672x8192x4 46 vs 62)
+    return p.M == 2 && mfma_min_rows() == 3 && (long)p.N * (p.K / 8) * p.nb <= (32l << 20);
 }
 
 template <int NB>

@@ -125,6 +125,23 @@ def _read_layer_file(path):
     return ckpt["bWeight"], ckpt["alpha"]
 
 
+def save_shiftaddllm_weight(weights_dir, model_name, layer_name, wbits, bWeight, alpha):
+    """Write one layer in the on-disk Lat. format the loaders read: a torch file
+    `{model_name}_{layer_name}_{wbits}bit.pt` holding `bWeight` int32 [K, N/32, wbits]
+    (signs packed along the OUTPUT axis) and `alpha` fp32 [K/8, R, wbits]
+    (quant_methods/shiftaddllm.py:193-211 writes these keys and this name;
+    `layer_name` is "<block index>.<module path>", e.g. "0.self_attn.q_proj").
+    Returns the path."""
+    if bWeight.dtype != torch.int32 or bWeight.dim() != 3 or bWeight.size(2) != wbits:
+        raise ValueError("bWeight must be int32 [K, N/32, wbits]")
+    if alpha.dim() != 3 or alpha.size(2) != wbits or alpha.size(0) * 8 != bWeight.size(0):
+        raise ValueError("alpha must be [K/8, R, wbits]")
+    os.makedirs(weights_dir, exist_ok=True)
+    path = _layer_file(weights_dir, model_name, layer_name, wbits)
+    torch.save({"bWeight": bWeight.cpu().contiguous(), "alpha": alpha.float().cpu().contiguous()}, path)
+    return path
+
+
 def dequantize_lat(BinaryWeight: torch.Tensor, alpha: torch.Tensor) -> torch.Tensor:
     """On-disk Lat. tensors -> dense W_q [N, K] fp32 (lut_gemm/kernel.py:101-106)."""
     return unpack_weight(BinaryWeight, alpha.repeat_interleave(8, dim=0)).transpose(0, 1).contiguous()

@@ -1,0 +1,123 @@
+"""On-disk Lat. checkpoint format: writer, dense loader, kernel loader (CPU part),
+and on the GPU the loaded LutLinear layers against the dense model."""
+import numpy as np
+import pytest
+import torch
+import torch.nn as nn
+
+import oracle as orc
+from shiftaddllm_amd import workload
+from shiftaddllm_amd.lut_gemm import kernel as K
+from shiftaddllm_amd.lut_gemm.quant import LutLinear
+
+
+class _Attn(nn.Module):
+    def __init__(self, h):
+        super().__init__()
+        self.q_proj = nn.Linear(h, h, bias=False)
+        self.o_proj = nn.Linear(h, h, bias=False)
+
+
+class _Mlp(nn.Module):
+    def __init__(self, h, i):
+        super().__init__()
+        self.up_proj = nn.Linear(h, i, bias=False)
+        self.down_proj = nn.Linear(i, h, bias=False)
+
+
+class _Block(nn.Module):
+    def __init__(self, h, i):
+        super().__init__()
+        self.self_attn = _Attn(h)
+        self.mlp = _Mlp(h, i)
+
+
+class _Inner(nn.Module):
+    def __init__(self, n, h, i):
+        super().__init__()
+        self.layers = nn.ModuleList(_Block(h, i) for _ in range(n))
+
+
+class TinyLlamaTree(nn.Module):
+    """`model.model.layers[i].{self_attn,mlp}.*_proj`, the module paths of a Llama checkpoint."""
+    def __init__(self, n=2, h=64, i=96):
+        super().__init__()
+        self.model = _Inner(n, h, i)
+
+
+def _write_checkpoint(tmp_path, model, wbits, R, seed=0):
+    want = {}
+    layers = model.model.layers
+    for i in range(len(layers)):
+        for name, lin in K.find_layers(layers[i], layers=(nn.Linear,)).items():
+            p = workload.make_block_problem(lin.out_features, lin.in_features, nb=wbits, R=R, seed=seed + 7 * i + len(name))
+            path = K.save_shiftaddllm_weight(str(tmp_path), "tiny", f"{i}.{name}", wbits, p.disk_bWeight, p.disk_alpha)
+            assert path.endswith(f"tiny_{i}.{name}_{wbits}bit.pt")
+            want[(i, name)] = orc.dequant_lat_disk(p.disk_bWeight.numpy(), p.disk_alpha.numpy())     # [N, K]
+    return want
+
+
+def test_writer_rejects_malformed_tensors(tmp_path):
+    bw = torch.zeros((64, 2, 3), dtype=torch.int32)
+    al = torch.ones((8, 4, 3))
+    with pytest.raises(ValueError):
+        K.save_shiftaddllm_weight(str(tmp_path), "m", "0.x", 2, bw, al)          # bit count mismatch
+    with pytest.raises(ValueError):
+        K.save_shiftaddllm_weight(str(tmp_path), "m", "0.x", 3, bw, al[:4])      # alpha rows != K/8
+    with pytest.raises(ValueError):
+        K.save_shiftaddllm_weight(str(tmp_path), "m", "0.x", 3, bw.long(), al)
+
+
+def test_dense_loader_round_trip(tmp_path):
+    model = TinyLlamaTree()
+    want = _write_checkpoint(tmp_path, model, wbits=3, R=4)
+    missing = K.load_shiftaddllm_weight(model, str(tmp_path), "tiny", 3, is_lat=True)
+    assert missing == []
+    for (i, name), W in want.items():
+        lin = K.find_layers(model.model.layers[i], layers=(nn.Linear,))[name]
+        assert np.array_equal(lin.weight.detach().numpy(), W.astype(np.float32))
+
+
+def test_dense_loader_reports_missing_files(tmp_path, capsys):
+    model = TinyLlamaTree(n=1)
+    missing = K.load_shiftaddllm_weight(model, str(tmp_path), "tiny", 3, is_lat=True)
+    assert len(missing) == 4 and "WARNING: no such file" in capsys.readouterr().out
+
+
+@pytest.mark.parametrize("alpha_format", ["apot_int8", "block_fp16"])
+def test_kernel_loader_fills_lutlinear_buffers(tmp_path, alpha_format):
+    model = TinyLlamaTree()
+    want = _write_checkpoint(tmp_path, model, wbits=2, R=4, seed=3)
+    missing = K.load_shiftaddllm_weight_with_kernel(model, str(tmp_path), "tiny", 2, is_lat=True,
+                                                    alpha_format=alpha_format)
+    assert missing == []
+    luts = K.find_layers(model.model.layers[0], layers=(LutLinear,))
+    assert set(luts) == {"self_attn.q_proj", "self_attn.o_proj", "mlp.up_proj", "mlp.down_proj"}
+    for (i, name), W in want.items():
+        lut = K.find_layers(model.model.layers[i], layers=(LutLinear,))[name]
+        assert lut.num_groups == 4 and lut.wbit == 2
+        bW = lut.binaryWeight.numpy()
+        if alpha_format == "apot_int8":
+            alpha = orc.apot_i8_to_alpha(lut.alpha.numpy())
+        else:
+            alpha = lut.alpha.numpy().astype(np.float32)
+        got = orc.dequant_block_kernel_layout(bW, alpha)
+        assert np.array_equal(got, W.astype(np.float32)), (i, name)
+
+
+@pytest.mark.gpu
+def test_loaded_layers_match_dense_layers_on_gpu(tmp_path, gpu_device):
+    dense, lut = TinyLlamaTree(h=128, i=256), TinyLlamaTree(h=128, i=256)
+    _write_checkpoint(tmp_path, dense, wbits=3, R=4, seed=5)
+    K.load_shiftaddllm_weight(dense, str(tmp_path), "tiny", 3, is_lat=True)
+    K.load_shiftaddllm_weight_with_kernel(lut, str(tmp_path), "tiny", 3, is_lat=True)
+    dense, lut = dense.to(gpu_device), lut.to(gpu_device)
+    x = torch.randn((1, 128), generator=torch.Generator().manual_seed(1)).half().to(gpu_device)
+    for i in range(2):
+        for name in ("self_attn.q_proj", "self_attn.o_proj", "mlp.up_proj"):
+            d = K.find_layers(dense.model.layers[i], layers=(nn.Linear,))[name]
+            l = K.find_layers(lut.model.layers[i], layers=(LutLinear,))[name]
+            want = (x.float() @ d.weight.float().t()).cpu().numpy()
+            got = l(x).float().cpu().numpy()
+            rel, mad = orc.error_metrics(got, want)
+            assert rel <= 2e-3 and mad <= 1e-2, (i, name, rel, mad)
