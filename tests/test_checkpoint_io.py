@@ -117,7 +117,7 @@ def test_loaded_layers_match_dense_layers_on_gpu(tmp_path, gpu_device):
         for name in ("self_attn.q_proj", "self_attn.o_proj", "mlp.up_proj"):
             d = K.find_layers(dense.model.layers[i], layers=(nn.Linear,))[name]
             l = K.find_layers(lut.model.layers[i], layers=(LutLinear,))[name]
-            want = (x.float() @ d.weight.float().t()).cpu().numpy()
-            got = l(x).float().cpu().numpy()
+            want = (x.float() @ d.weight.detach().float().t()).cpu().numpy()
+            got = l(x).detach().float().cpu().numpy()
             rel, mad = orc.error_metrics(got, want)
             assert rel <= 2e-3 and mad <= 1e-2, (i, name, rel, mad)
