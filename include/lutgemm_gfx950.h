@@ -147,7 +147,10 @@ size_t lutgemm_algorithmic_bytes(int N, int K, int nb, int M, size_t alpha_entri
 int lutgemm_copy_bytes(void *dst, const void *src, size_t bytes, void *stream);
 
 /* Release the per-stream workspaces this library allocated on the current
- * device (optional; they otherwise live until the process ends). */
+ * device (optional; they otherwise live until the process ends).  HIP graphs
+ * captured from calls of this library name those workspaces: destroy such
+ * graphs first.  A workspace that a later, larger call outgrew is kept until
+ * this call for the same reason. */
 int lutgemm_release_workspaces(void);
 
 /*

@@ -47,6 +47,7 @@
 #include <mutex>
 #include <type_traits>
 #include <utility>
+#include <vector>
 
 #include "lutgemm_gfx950.h"
 #include "lutgemm_internal.h"
@@ -1006,6 +1007,7 @@ thread_local int g_last_hip_error = 0;
 struct Workspace {
     unsigned long long *accum = nullptr;
     size_t words = 0;
+    std::vector<unsigned long long *> retired;  // outgrown buffers: captured graphs may still name them
 };
 
 std::mutex g_ws_mutex;
@@ -1020,7 +1022,9 @@ int hip_fail(hipError_t e)
 // Grow-only, zero-initialised accumulator words per (device, stream).  Launches
 // on one stream are ordered and every launch leaves its words at zero again, so
 // a stream shares one workspace across calls.  Growing synchronises the stream
-// and allocates: do a first call of each shape before capturing a graph.
+// and allocates: do a first call of each shape before capturing a graph.  An
+// outgrown buffer is kept (zero, unused by new launches) until
+// lutgemm_release_workspaces(): a graph captured earlier still points at it.
 int get_workspace(hipStream_t stream, size_t words, unsigned long long **out)
 {
     int dev = 0;
@@ -1031,7 +1035,7 @@ int get_workspace(hipStream_t stream, size_t words, unsigned long long **out)
     if (ws.words < words) {
         e = hipStreamSynchronize(stream);  // queued work may still use the old buffer
         if (e != hipSuccess) return hip_fail(e);
-        if (ws.accum) (void)hipFree(ws.accum);
+        if (ws.accum) ws.retired.push_back(ws.accum);
         ws.accum = nullptr;
         ws.words = 0;
         size_t want = words < (1u << 18) ? (1u << 18) : words;
@@ -1528,6 +1532,7 @@ int lutgemm_release_workspaces(void)
     for (auto it = g_workspaces.begin(); it != g_workspaces.end();) {
         if (it->first.first == dev) {
             if (it->second.accum) (void)hipFree(it->second.accum);
+            for (unsigned long long *old : it->second.retired) (void)hipFree(old);
             it = g_workspaces.erase(it);
         } else {
             ++it;

@@ -474,3 +474,39 @@ def test_decoder_matches_dense_dequantised_model(gpu_device):
     r2 = decode.benchmark(lut, ids, generate=4, warmup=1)
     assert r1["generated"].shape == (2, 4) and torch.equal(r1["generated"], r2["generated"])
     assert r1["median_s_per_token"] > 0
+
+
+def test_captured_graph_survives_workspace_growth(gpu_device):
+    """A graph captured on a stream keeps working after a larger problem on the same
+    stream made the library outgrow the K-split workspace the graph points at."""
+    lib = native.cabi()
+    small = workload.make_rowwise_problem(512, 1024, nb=3, M=1, seed=21, device=gpu_device, quantize=False)
+    big = workload.make_rowwise_problem(8192, 1024, nb=2, M=40, seed=22, device=gpu_device, quantize=False)
+    want, _ = orc.gemv_rowwise_c(small.bW.cpu().numpy(), small.alpha.cpu().numpy(), small.x.cpu().numpy(),
+                                 small.num_groups)
+    stream = torch.cuda.Stream()
+    sp = ctypes.c_void_p(stream.cuda_stream)
+    out = torch.zeros((1, 512), dtype=torch.float16, device=gpu_device)
+    p = lambda t: ctypes.c_void_p(t.data_ptr())
+
+    def call(pr, o):
+        rc = lib.lutgemm_gemv_rowwise_f16(p(pr.bW), p(pr.alpha), p(pr.x), p(o), pr.N, pr.K, pr.nb, pr.num_groups,
+                                          pr.x.shape[0], sp)
+        assert rc == 0, lib.lutgemm_strerror(rc).decode()
+
+    with torch.cuda.stream(stream):
+        call(small, out)                                  # sizes the stream's workspace
+    stream.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=stream):
+        call(small, out)
+    big_out = torch.zeros((40, 8192), dtype=torch.float16, device=gpu_device)
+    with torch.cuda.stream(stream):
+        call(big, big_out)                                # 40 x 8192 words: larger than the first allocation
+    stream.synchronize()
+    for _ in range(3):
+        with torch.cuda.stream(stream):
+            out.zero_()
+            graph.replay()
+        stream.synchronize()
+        _assert_close(out, want, "replay after growth")
