@@ -768,29 +768,33 @@ constexpr int kMfmaTileCols = 64;     // outputs per workgroup
 constexpr int kMfmaStepK = 128;
 constexpr int kXRowBytes = 256 + 16;  // one activation row of a K-step, padded against bank conflicts
 
+constexpr int kAlphaStepHalves = 64;  // alphas of one (K-step, bit plane): the workgroup's 64 outputs
+
+// Sign words of one K-step of a wave: word kb of 4 outputs per bit plane.
 template <int NB>
-struct MfmaOperands {
-    u32x4 w[NB];      // sign words of 4 outputs
-    u32x2 a[NB][4];   // 16 fp16 alphas: outputs base + 16*kb .. +15
+struct MfmaSigns {
+    u32x4 w[NB];
 };
 
 template <int NB>
-__device__ __forceinline__ void mfma_load_step(MfmaOperands<NB> &r, const Problem &p, int step, int kb,
-                                               uint32_t wcol4, uint32_t acol2)
+__device__ __forceinline__ void mfma_load_signs(MfmaSigns<NB> &r, const Problem &p, int step, int kb, uint32_t wcol4)
 {
     const uint32_t row_bytes = (uint32_t)p.N * 4u;
     const char *wbase = (const char *)p.W + (size_t)step * 4 * NB * row_bytes;
     const uint32_t wrow = (uint32_t)kb * (NB * row_bytes);
-    const int g = (step * 4) / p.group_words;
-    const uint32_t arow = (uint32_t)g * (NB * (uint32_t)p.N * 2u);
 #pragma unroll
-    for (int b = 0; b < NB; ++b) {
+    for (int b = 0; b < NB; ++b)
         r.w[b] = __builtin_nontemporal_load((const u32x4 *)(wbase + (size_t)b * row_bytes + (wrow + wcol4)));
-        const char *asrc = (const char *)p.alpha + (size_t)b * p.N * 2u + (arow + acol2);
-#pragma unroll
-        for (int v = 0; v < 4; ++v) r.a[b][v] = *(const u32x2 *)(asrc + 8 * v);
-    }
 }
+
+// What a thread fetches for the staging of one round (8 K-steps): 4*MT activation
+// targets (16 bytes each after the shuffle into MFMA K order) and one 8-byte run of
+// alphas.
+template <int MT>
+struct MfmaStage {
+    u32x2 lo[4 * MT], hi[4 * MT];
+    u32x2 alpha;
+};
 
 // 8 signs of sign word `w` -> 8 fp16 +-1.0 (bit set = +1.0): pair i holds
 // bit 4*beta+i (low half) and bit 16+4*beta+i (high half).
@@ -808,7 +812,8 @@ __device__ __forceinline__ f16x8 expand_signs(uint32_t w, int beta)
 }
 
 // xs: activations of one round, [wave's step][row][word][instance][8 halves],
-// kMfmaWaves * 16 * MT * kXRowBytes bytes; reused for the final reduction.
+// kMfmaWaves * 16 * MT * kXRowBytes bytes (reused for the final reduction), followed
+// by the alphas of the round, kMfmaWaves * NB * 64 halves.
 template <int NB, int MT>
 __device__ __forceinline__ void mfma_tile(const Problem &p, int local_block, char *xs)
 {
@@ -825,28 +830,55 @@ __device__ __forceinline__ void mfma_tile(const Problem &p, int local_block, cha
     const int n_base = tile * kMfmaTileCols;
 
     const uint32_t wcol4 = (uint32_t)min(n_base + 4 * li, p.N - 4) * 4u;
-    const uint32_t acol2 = (uint32_t)min(n_base + 16 * kb, p.N - 16) * 2u;
 
     const int step_begin = kslice * p.sets_per_split;
     const int step_end = min(step_begin + p.sets_per_split, p.nsets);
 
-    // Stage the activations of the round starting at step r0: target t = (step s of
-    // the round, row rr, word w, instance beta) gets 8 halves in MFMA K order.
-    auto stage_round = [&](int r0) {
+    // Staging of a round (8 K-steps, one per wave), fetched one round ahead into
+    // registers and written to LDS between two barriers:
+    //  * activations: target t = (step s of the round, row rr, word w, instance beta)
+    //    gets 8 halves in MFMA K order;
+    //  * alphas: thread t < 128*NB fetches alpha[group of step s][plane b][base + 4q .. +3]
+    //    (s, b, q from t) and scatters it to as[s][b][kb][e][r], so that a lane reads
+    //    the four alphas of its D rows (one e, r = 0..3) as one 8-byte word.
+    char *as = xs + kMfmaWaves * kWaveXBytes;
+    const int a_q = tid & 15, a_sb = tid >> 4;          // alpha role: 4 outputs 4q.., (step, plane)
+    const int a_s = a_sb / NB, a_b = a_sb % NB;
+    const bool a_role = tid < 16 * kMfmaWaves * NB;
+    const uint32_t acol2 = (uint32_t)min(n_base + 4 * a_q, p.N - 4) * 2u;
+
+    auto fetch_stage = [&](MfmaStage<MT> &st, int r0) {
 #pragma unroll
         for (int u = 0; u < 4 * MT; ++u) {
             const int t = tid + kMfmaThreads * u;
             const int beta = t & 3, w = (t >> 2) & 3, rr = (t >> 4) % (16 * MT), sidx = t / (256 * MT);
             const int step = min(r0 + sidx, p.nsets - 1);
             const __half *src = p.x + (size_t)min(m0 + rr, p.M - 1) * p.K + step * kMfmaStepK + 32 * w + 4 * beta;
-            const u32x2 lo = *(const u32x2 *)src;
-            const u32x2 hi = *(const u32x2 *)(src + 16);
+            st.lo[u] = *(const u32x2 *)src;
+            st.hi[u] = *(const u32x2 *)(src + 16);
+        }
+        const int g = (min(r0 + (a_role ? a_s : 0), p.nsets - 1) * 4) / p.group_words;
+        st.alpha = *(const u32x2 *)((const char *)p.alpha + ((size_t)g * NB + (a_role ? a_b : 0)) * p.N * 2u + acol2);
+    };
+    auto store_stage = [&](const MfmaStage<MT> &st) {
+#pragma unroll
+        for (int u = 0; u < 4 * MT; ++u) {
+            const int t = tid + kMfmaThreads * u;
+            const int beta = t & 3, w = (t >> 2) & 3, rr = (t >> 4) % (16 * MT), sidx = t / (256 * MT);
             u32x4 v;
-            v.x = __builtin_amdgcn_perm(hi.x, lo.x, 0x05040100u);
-            v.y = __builtin_amdgcn_perm(hi.x, lo.x, 0x07060302u);
-            v.z = __builtin_amdgcn_perm(hi.y, lo.y, 0x05040100u);
-            v.w = __builtin_amdgcn_perm(hi.y, lo.y, 0x07060302u);
+            v.x = __builtin_amdgcn_perm(st.hi[u].x, st.lo[u].x, 0x05040100u);
+            v.y = __builtin_amdgcn_perm(st.hi[u].x, st.lo[u].x, 0x07060302u);
+            v.z = __builtin_amdgcn_perm(st.hi[u].y, st.lo[u].y, 0x05040100u);
+            v.w = __builtin_amdgcn_perm(st.hi[u].y, st.lo[u].y, 0x07060302u);
             *(u32x4 *)(xs + sidx * kWaveXBytes + rr * kXRowBytes + w * 64 + beta * 16) = v;
+        }
+        if (a_role) {
+            // outputs 4q + e, e = 0..3: kb = q >> 2, r = q & 3
+            unsigned short *dst = (unsigned short *)as + ((a_s * NB + a_b) * 4 + (a_q >> 2)) * 16 + (a_q & 3);
+            dst[0] = (unsigned short)(st.alpha.x & 0xffffu);
+            dst[4] = (unsigned short)(st.alpha.x >> 16);
+            dst[8] = (unsigned short)(st.alpha.y & 0xffffu);
+            dst[12] = (unsigned short)(st.alpha.y >> 16);
         }
     };
 
@@ -856,8 +888,9 @@ __device__ __forceinline__ void mfma_tile(const Problem &p, int local_block, cha
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) acc[e][mt] = (f32x4){0.0f, 0.0f, 0.0f, 0.0f};
 
-    auto compute = [&](const MfmaOperands<NB> &ops) {
+    auto compute = [&](const MfmaSigns<NB> &ops) {
         const char *xw = xs + wave * kWaveXBytes;
+        const u32x2 *aw = (const u32x2 *)as + (wave * NB * 4 + kb) * 4;   // + b*16 + e
         f16x8 bx[MT][4];
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt)
@@ -869,6 +902,7 @@ __device__ __forceinline__ void mfma_tile(const Problem &p, int local_block, cha
             const uint32_t w4[4] = {ops.w[b].x, ops.w[b].y, ops.w[b].z, ops.w[b].w};
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
+                const u32x2 al = aw[b * 16 + e];  // alphas of D rows r = 0..3 (outputs base + 16*kb + 4*r + e)
                 f32x4 d[MT];
 #pragma unroll
                 for (int mt = 0; mt < MT; ++mt) d[mt] = (f32x4){0.0f, 0.0f, 0.0f, 0.0f};
@@ -879,30 +913,43 @@ __device__ __forceinline__ void mfma_tile(const Problem &p, int local_block, cha
                     for (int mt = 0; mt < MT; ++mt)
                         d[mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, bx[mt][beta], d[mt], 0, 0, 0);
                 }
-                // D row 4*kb + r is output base + 16*kb + 4*r + e: alpha number 4*r + e of the lane's 16
+                const uint32_t araw[4] = {al.x & 0xffffu, al.x >> 16, al.y & 0xffffu, al.y >> 16};
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
-                    const int idx = 4 * r + e;
-                    const uint32_t raw = (idx & 2) ? ops.a[b][idx >> 2].y : ops.a[b][idx >> 2].x;
-                    const float al = half_bits_to_float((raw >> (16 * (idx & 1))) & 0xffffu);
+                    const float alr = half_bits_to_float(araw[r]);
 #pragma unroll
-                    for (int mt = 0; mt < MT; ++mt) acc[e][mt][r] = fmaf(d[mt][r], al, acc[e][mt][r]);
+                    for (int mt = 0; mt < MT; ++mt) acc[e][mt][r] = fmaf(d[mt][r], alr, acc[e][mt][r]);
                 }
             }
         }
     };
 
-    // rounds of 8 steps, one per wave; the next round's sign words are already in
-    // flight while the activations are staged
-    MfmaOperands<NB> ops;
-    for (int r0 = step_begin; r0 < step_end; r0 += kMfmaWaves) {
-        const int step = r0 + wave;
-        const bool live = step < step_end;
-        mfma_load_step<NB>(ops, p, min(step, p.nsets - 1), kb, wcol4, acol2);
-        __syncthreads();  // previous round's readers are done with xs
-        stage_round(r0);
+    // Rounds of 8 steps, one per wave, software pipelined: while round i is
+    // multiplied, the sign words of round i+1 (the HBM stream) are in flight; two sign
+    // buffers alternate (no register copies) and loads are clamped, not predicated, so
+    // that the waits can count them.  The staging data (activations and alphas, L2
+    // hits) is fetched a round ahead too where registers allow: in the 32-row tile,
+    // which has one workgroup per CU anyway.  The 16-row tile keeps to 128 registers
+    // so that two workgroups share a CU (measured, 28672x8192x4: 62 us with two
+    // resident workgroups and no look-ahead, 70-74 us with one and full look-ahead).
+    constexpr bool kStageAhead = MT == 2 && NB >= 3;
+    MfmaSigns<NB> sgA, sgB;
+    MfmaStage<MT> st;
+    mfma_load_signs<NB>(sgA, p, min(step_begin + wave, p.nsets - 1), kb, wcol4);
+    if constexpr (kStageAhead) fetch_stage(st, step_begin);
+    // (the look-ahead of the last round re-reads clamped addresses and is discarded)
+    auto round = [&](const MfmaSigns<NB> &cur, MfmaSigns<NB> &nxt, int r0) {
+        __syncthreads();  // the previous round's readers are done with the staged data
+        if constexpr (!kStageAhead) fetch_stage(st, r0);
+        store_stage(st);
+        mfma_load_signs<NB>(nxt, p, min(r0 + kMfmaWaves + wave, p.nsets - 1), kb, wcol4);
+        if constexpr (kStageAhead) fetch_stage(st, r0 + kMfmaWaves);
         __syncthreads();
-        if (live) compute(ops);
+        if (r0 + wave < step_end) compute(cur);
+    };
+    for (int r0 = step_begin; r0 < step_end; r0 += 2 * kMfmaWaves) {
+        round(sgA, sgB, r0);
+        if (r0 + kMfmaWaves < step_end) round(sgB, sgA, r0 + kMfmaWaves);
     }
 
     // ---- the 8 waves' accumulators meet in LDS -----------------------------------
@@ -968,7 +1015,7 @@ __device__ __forceinline__ void mfma_tile(const Problem &p, int local_block, cha
 template <int NB, int MT>
 __global__ void __launch_bounds__(kMfmaThreads) lut_gemm_mfma_kernel(const Problem p)
 {
-    __shared__ __attribute__((aligned(16))) char xs[kMfmaWaves * 16 * MT * kXRowBytes];
+    __shared__ __attribute__((aligned(16))) char xs[kMfmaWaves * 16 * MT * kXRowBytes + kMfmaWaves * NB * kAlphaStepHalves * 2];
     mfma_tile<NB, MT>(p, (int)blockIdx.x, xs);
 }
 
@@ -976,7 +1023,7 @@ __global__ void __launch_bounds__(kMfmaThreads) lut_gemm_mfma_kernel(const Probl
 template <int MT>
 __global__ void __launch_bounds__(kMfmaThreads) lut_gemm_mfma_group_kernel(const Group g)
 {
-    __shared__ __attribute__((aligned(16))) char xs[kMfmaWaves * 16 * MT * kXRowBytes];
+    __shared__ __attribute__((aligned(16))) char xs[kMfmaWaves * 16 * MT * kXRowBytes + kMfmaWaves * 4 * kAlphaStepHalves * 2];
     const int b = blockIdx.x;
     int pi = 0;
 #pragma unroll
