@@ -51,6 +51,8 @@ def parse_args():
                     help="only the 224-launch step (no fused sequences, no per-shape table): for profiler runs")
     ap.add_argument("--profile-shape", type=str, default="",
                     help="N,K[,nb[,iters[,M]]]: only launch this shape repeatedly (for rocprofv3 runs) and exit")
+    ap.add_argument("--batch-table", action="store_true",
+                    help="only time the 70B and 7B shapes over 1..32 activation rows (graph replay, rotating weights) and exit")
     ap.add_argument("--profile-decode", type=int, default=0,
                     help="batch: only replay ten graph-captured decode steps of the 7B decoder (for rocprofv3 runs) and exit")
     ap.add_argument("--profile-copy", type=int, default=0,
@@ -118,6 +120,43 @@ def main():
                 lib.lutgemm_copy_bytes(ctypes.c_void_p(dst.data_ptr()), ctypes.c_void_p(src.data_ptr()), nbytes, sp)
         stream.synchronize()
         print(json.dumps({"copy_bytes": nbytes, "launches": 5}))
+        return
+    if args.batch_table:
+        import statistics
+        table = {}
+        shapes = [(8192, 8192, 2), (8192, 8192, 4), (28672, 8192, 2), (28672, 8192, 4), (8192, 28672, 4),
+                  (1024, 8192, 4), (4096, 4096, 3)]
+        for (N, K, nb) in shapes:
+            row = {}
+            for M in (1, 2, 4, 8, 16, 32):
+                cnt = max(3, min(24, (400 << 20) // (K // 8 * N * nb)))     # distinct weight sets: > 256 MB in rotation
+                pool = [Gemv(torch, dev, N, K, nb, 7 * i + M, M=M) for i in range(cnt)]
+                with torch.cuda.stream(stream):
+                    run(pool[0], sp)                                         # sizes the stream's workspace
+                stream.synchronize()
+                seq = (pool * ((24 + cnt - 1) // cnt))[:max(24, cnt)]
+                gr = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(gr, stream=stream):
+                    for g in seq:
+                        run(g, sp)
+                ts = []
+                for _ in range(3):
+                    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                    with torch.cuda.stream(stream):
+                        e0.record(stream)
+                        gr.replay()
+                        e1.record(stream)
+                    torch.cuda.synchronize()
+                    ts.append(e0.elapsed_time(e1) * 1e3 / len(seq))
+                us = statistics.median(ts)
+                byts = lib.lutgemm_algorithmic_bytes(N, K, nb, M, (K // GROUP) * nb * N, 2)
+                row[f"M{M}"] = {"us_per_call": round(us, 1), "GBps": round(byts / us / 1e3),
+                                "dense_equiv_TFLOPs": round(2 * M * N * K / us / 1e6, 1)}
+                del pool, seq, gr
+            table[f"{N}x{K}x{nb}bit"] = row
+        print(json.dumps({"batch_table": table, "note": "one launch per call, HIP-graph replay of 24 calls over "
+                          "rotating weights, median of 3; 1 row (and 2 rows above 32 MB of signs) = table look-up "
+                          "kernel, otherwise matrix-core kernel"}))
         return
     if args.profile_decode:
         from shiftaddllm_amd import decode
