@@ -81,8 +81,27 @@ rmsnorm_kernel(const __half *__restrict__ x, const __half *__restrict__ w, __hal
     const u32x4 *wr = (const u32x4 *)w;
     u32x4 *yr = (u32x4 *)(y + (size_t)r * hidden);
     const int chunks = hidden / 8;
+    // the first kHeld chunks of a thread stay in registers, with the matching weights,
+    // so that rows up to 8192 wide cost one memory round trip
+    constexpr int kHeld = 4;
+    u32x4 xv[kHeld], wv[kHeld];
+#pragma unroll
+    for (int u = 0; u < kHeld; ++u) {
+        const int c = min(tid + kThreads * u, chunks - 1);
+        xv[u] = xr[c];
+        wv[u] = wr[c];
+    }
     float ss = 0.0f;
-    for (int c = tid; c < chunks; c += kThreads) {
+#pragma unroll
+    for (int u = 0; u < kHeld; ++u) {
+        if (tid + kThreads * u < chunks) {
+            float f[8];
+            unpack8(xv[u], f);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) ss = fmaf(f[i], f[i], ss);
+        }
+    }
+    for (int c = tid + kThreads * kHeld; c < chunks; c += kThreads) {
         float f[8];
         unpack8(xr[c], f);
 #pragma unroll
@@ -90,10 +109,10 @@ rmsnorm_kernel(const __half *__restrict__ x, const __half *__restrict__ w, __hal
     }
     ss = block_reduce<false>(ss, red);
     const float scale = rsqrtf(ss / (float)hidden + eps);
-    for (int c = tid; c < chunks; c += kThreads) {
+    auto finish = [&](const u32x4 &xc, const u32x4 &wc) {
         float f[8], g[8];
-        unpack8(xr[c], f);
-        unpack8(wr[c], g);
+        unpack8(xc, f);
+        unpack8(wc, g);
         u32x4 o;
         uint32_t *ow = (uint32_t *)&o;
 #pragma unroll
@@ -102,8 +121,12 @@ rmsnorm_kernel(const __half *__restrict__ x, const __half *__restrict__ w, __hal
             const float b = __half2float(__float2half_rn(f[2 * i + 1] * scale)) * g[2 * i + 1];
             ow[i] = pack2(a, b);
         }
-        yr[c] = o;
-    }
+        return o;
+    };
+#pragma unroll
+    for (int u = 0; u < kHeld; ++u)
+        if (tid + kThreads * u < chunks) yr[tid + kThreads * u] = finish(xv[u], wv[u]);
+    for (int c = tid + kThreads * kHeld; c < chunks; c += kThreads) yr[c] = finish(xr[c], wr[c]);
 }
 
 // One workgroup per (sequence b, query head h).  Rotates q and the new k by the
