@@ -122,7 +122,6 @@ def main():
         print(json.dumps({"copy_bytes": nbytes, "launches": 5}))
         return
     if args.batch_table:
-        import statistics
         table = {}
         shapes = [(8192, 8192, 2), (8192, 8192, 4), (28672, 8192, 2), (28672, 8192, 4), (8192, 28672, 4),
                   (1024, 8192, 4), (4096, 4096, 3)]
