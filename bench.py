@@ -396,8 +396,8 @@ def main():
                                 f"random.Random(0) ({counts[2]}x2-bit, {counts[3]}x3-bit, {counts[4]}x4-bit), "
                                 "group 128, 128 prompt tokens fed one by one then 128 greedy tokens, one "
                                 "HIP-graph replay + sync per token; q/k/v and gate/up as grouped launches; "
-                                "batch 1: RMSNorm and SiLU*up folded into the look-up GEMVs, rotary + KV append "
-                                "+ attention in one HIP kernel (5 launches per block); batch 8: matrix-core "
+                                "batch 1: SiLU*up folded into the down_proj look-up GEMV, RMSNorm and rotary + KV "
+                                "append + attention as one HIP kernel each (7 launches per block); batch 8: matrix-core "
                                 "GEMM kernel with RMSNorm / attention / SiLU*up HIP kernels between (8 launches "
                                 "per block); embedding gather and fp16 lm_head in torch")
 
