@@ -69,7 +69,7 @@ int lutgemm_gemv_rowwise_f16(const uint32_t *bW, const void *alpha_f16, const vo
  * a 7B-sized GEMV needs at HBM speed, so projections that do not depend on each
  * other (q/k/v, gate/up) are best issued together.  Each entry has the
  * arguments and the semantics of lutgemm_gemv_rowwise_f16; bit widths and
- * shapes may differ between entries, outputs must not overlap.
+ * shapes may differ between entries; outputs must not overlap (LUTGEMM_EINVAL).
  * 1 <= count <= LUTGEMM_MAX_GROUP.
  */
 #define LUTGEMM_MAX_GROUP 8

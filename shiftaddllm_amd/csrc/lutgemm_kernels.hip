@@ -1405,6 +1405,14 @@ int run_group(int count, const lutgemm_fused_problem *problems, hipStream_t stre
         words += (size_t)q.M * q.N;
         total_bytes += (long)q.N * (q.K / 8) * q.nb * q.M;
     }
+    // every problem finishes its outputs with a plain read-modify-write: two problems
+    // of one launch may not write the same memory
+    for (int i = 0; i < count; ++i)
+        for (int j = i + 1; j < count; ++j) {
+            const char *a0 = (const char *)g.p[i].out, *a1 = a0 + (size_t)g.p[i].M * g.p[i].N * 2;
+            const char *b0 = (const char *)g.p[j].out, *b1 = b0 + (size_t)g.p[j].M * g.p[j].N * 2;
+            if (a0 < b1 && b0 < a1) return LUTGEMM_EINVAL;
+        }
     if (plain && all_mfma) {
         bool same_height = true;
         for (int i = 1; i < count; ++i) same_height = same_height && ((g.p[i].M > 16) == (g.p[0].M > 16));

@@ -510,3 +510,18 @@ def test_captured_graph_survives_workspace_growth(gpu_device):
             graph.replay()
         stream.synchronize()
         _assert_close(out, want, "replay after growth")
+
+
+def test_grouped_launch_rejects_overlapping_outputs(gpu_device):
+    lib = native.cabi()
+    a = workload.make_rowwise_problem(256, 256, nb=2, seed=1, device=gpu_device, quantize=False)
+    out = torch.zeros((1, 512), dtype=torch.float16, device=gpu_device)
+    arr = (native.RowwiseProblem * 2)()
+    for i, off in enumerate((0, 128)):                      # second output starts inside the first
+        arr[i] = native.RowwiseProblem(a.bW.data_ptr(), a.alpha.data_ptr(), a.x.data_ptr(), out.data_ptr() + 2 * off,
+                                       256, 256, 2, a.num_groups, 1)
+    assert lib.lutgemm_gemv_rowwise_f16_grouped(2, arr, _stream()) == -1
+    arr[1].out_f16 = out.data_ptr() + 2 * 256               # adjacent is fine
+    assert lib.lutgemm_gemv_rowwise_f16_grouped(2, arr, _stream()) == 0
+    torch.cuda.synchronize()
+    assert torch.equal(out[:, :256], out[:, 256:])
