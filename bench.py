@@ -153,7 +153,60 @@ def main():
                                 "dense_equiv_TFLOPs": round(2 * M * N * K / us / 1e6, 1)}
                 del pool, seq, gr
             table[f"{N}x{K}x{nb}bit"] = row
-        print(json.dumps({"batch_table": table, "note": "one launch per call, HIP-graph replay of 24 calls over "
+        # config 3: Llama-2-13B shapes, 2-bit, block alpha (8 row groups), one row, every storage format
+        block = {}
+        entry = {"f16": lib.lutgemm_gemv_block_f16, "apot_i8": lib.lutgemm_gemv_block_apot_i8,
+                 "shift_u16": lib.lutgemm_gemv_block_shift_u16}
+        vp = lambda t: ctypes.c_void_p(t.data_ptr())
+        for (N, K) in workload.LLAMA2_13B_SHAPES:
+            nb, R = 2, 8
+            row = {}
+            for kind, fn in entry.items():
+                cnt = max(4, min(40, (500 << 20) // (K // 8 * N * nb)))
+                pool = []
+                for i in range(cnt):
+                    g = torch.Generator(device=dev).manual_seed(17 * i + N)
+                    bW = torch.randint(-2 ** 31, 2 ** 31 - 1, (K // 32, nb, N), generator=g, device=dev, dtype=torch.int32)
+                    e = (torch.randint(-9, -5, (K // 8, 1, R), generator=g, device=dev).float()
+                         - torch.arange(nb, device=dev).float().view(1, nb, 1))
+                    if kind == "f16":
+                        alpha = torch.exp2(e).half().contiguous()
+                    elif kind == "apot_i8":
+                        alpha = torch.full((K // 8, nb, R, 3), -128, dtype=torch.int8, device=dev)
+                        alpha[..., 0] = e.to(torch.int8)
+                    else:
+                        alpha = torch.randint(0, 512, (K // 8, nb, R), generator=g, device=dev).to(torch.int16)
+                    pool.append((bW, alpha, torch.randn((1, K), generator=g, device=dev).half(),
+                                 torch.zeros((1, N), dtype=torch.float16, device=dev)))
+
+                def go(o, fn=fn, kind=kind, N=N, K=K):
+                    extra = () if kind == "f16" else (3,)
+                    rc = fn(vp(o[0]), vp(o[1]), vp(o[2]), vp(o[3]), N, K, nb, R, *extra, 1, sp)
+                    if rc:
+                        raise RuntimeError(lib.lutgemm_strerror(rc).decode())
+                with torch.cuda.stream(stream):
+                    go(pool[0])
+                stream.synchronize()
+                seq = (pool * 3)[:max(40, cnt)]
+                gr = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(gr, stream=stream):
+                    for o in seq:
+                        go(o)
+                ts = []
+                for _ in range(3):
+                    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                    with torch.cuda.stream(stream):
+                        e0.record(stream)
+                        gr.replay()
+                        e1.record(stream)
+                    torch.cuda.synchronize()
+                    ts.append(e0.elapsed_time(e1) * 1e3 / len(seq))
+                us = statistics.median(ts)
+                byts = lib.lutgemm_algorithmic_bytes(N, K, nb, 1, pool[0][1].numel(), pool[0][1].element_size())
+                row[kind] = {"us_per_call": round(us, 2), "GBps": round(byts / us / 1e3)}
+                del pool, seq, gr
+            block[f"{N}x{K}x{nb}bit_R{R}"] = row
+        print(json.dumps({"batch_table": table, "block_alpha_13b": block, "note": "one launch per call, HIP-graph replay of 24 calls over "
                           "rotating weights, median of 3; 1 row (and 2 rows above 32 MB of signs) = table look-up "
                           "kernel, otherwise matrix-core kernel"}))
         return
