@@ -124,7 +124,7 @@ def main():
     if args.batch_table:
         table = {}
         shapes = [(8192, 8192, 2), (8192, 8192, 4), (28672, 8192, 2), (28672, 8192, 4), (8192, 28672, 4),
-                  (1024, 8192, 4), (4096, 4096, 3)]
+                  (1024, 8192, 4), (4096, 4096, 3), (3072, 768, 3)]     # last: OPT-125m fc1 (config 1)
         for (N, K, nb) in shapes:
             row = {}
             for M in (1, 2, 4, 8, 16, 32):
