@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the LUT-GEMM hot path on one MI355X.
 
-Workload (BASELINE.json configs[1]): the seven linear layers of a Llama-2-7B
+Workload (the configuration the headline metric is quoted on): the seven linear layers of a Llama-2-7B
 decoder block as 3-bit BCQ LUT-GEMVs (group 128 along K, power-of-two alphas,
 batch 1).  One *step* is one decoded token's worth of them: 32 blocks x 7
 GEMVs = 224 launches streaming 2.74 GB of distinct weights (so nothing is
