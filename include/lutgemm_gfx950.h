@@ -167,8 +167,10 @@ int lutgemm_release_workspaces(void);
  *                     (out need not be initialised).
  * A problem with none of the three is the plain row-wise GEMV.  The problems of
  * one call must share their transform (all norm, all gate or all none;
- * LUTGEMM_EUNSUP otherwise).  Problems with a transform or with overwrite run on
- * the look-up kernel, whatever M.
+ * LUTGEMM_EUNSUP otherwise).  Problems with a transform always run on the
+ * look-up kernel, whatever M (with several rows a separate transform kernel in
+ * front of a plain call is faster); overwriting problems with several rows take
+ * the matrix-core kernel like plain ones.
  */
 typedef struct lutgemm_fused_problem {
     const uint32_t *bW;

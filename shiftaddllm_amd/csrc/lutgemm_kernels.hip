@@ -1001,13 +1001,13 @@ __device__ __forceinline__ void mfma_tile(const Problem &p, int local_block, cha
         if (m >= p.M || n >= p.N) continue;
         __half *dst = p.out + (size_t)m * p.N + n;
         if (p.ksplit == 1) {
-            *dst = __float2half_rn(__half2float(*dst) + val[i]);
+            *dst = __float2half_rn((p.overwrite ? 0.0f : __half2float(*dst)) + val[i]);
             continue;
         }
         if ((int)(old[i] >> 56) != p.ksplit - 1) continue;
         const long long total = (long long)((old[i] + contrib[i]) & kSumMask) - (long long)p.ksplit * kBias;
         const float y = (float)((double)total * (1.0 / 4294967296.0));
-        *dst = __float2half_rn(__half2float(*dst) + y);
+        *dst = __float2half_rn((p.overwrite ? 0.0f : __half2float(*dst)) + y);
         __hip_atomic_store(p.accum + (size_t)m * p.N + n, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
 }
@@ -1413,10 +1413,14 @@ int run_group(int count, const lutgemm_fused_problem *problems, hipStream_t stre
             const char *b0 = (const char *)g.p[j].out, *b1 = b0 + (size_t)g.p[j].M * g.p[j].N * 2;
             if (a0 < b1 && b0 < a1) return LUTGEMM_EINVAL;
         }
+    // The matrix-core kernel takes plain and (as a group launch) overwriting problems.
+    // Input transforms stay with the look-up kernel: there a workgroup transforms only
+    // its K-slice of one row, while every 64-output workgroup of the matrix-core kernel
+    // would redo the transform of all rows (measured slower than a separate kernel).
+    bool same_height = true;
+    for (int i = 1; i < count; ++i) same_height = same_height && ((g.p[i].M > 16) == (g.p[0].M > 16));
+    if (all_mfma && xform == kXNone && same_height && (count > 1 || !plain)) return run_mfma_group(g, stream);
     if (plain && all_mfma) {
-        bool same_height = true;
-        for (int i = 1; i < count; ++i) same_height = same_height && ((g.p[i].M > 16) == (g.p[0].M > 16));
-        if (count > 1 && same_height) return run_mfma_group(g, stream);
         for (int i = 0; i < count; ++i) {
             int rc = run_mfma(g.p[i], stream);
             if (rc != LUTGEMM_OK) return rc;

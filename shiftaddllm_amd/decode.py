@@ -223,14 +223,17 @@ class LutDecoder(nn.Module):
         q, k, v = self.qkv[:nq], self.qkv[nq:nq + nkv], self.qkv[nq + nkv:]
         g, u = self.gate_up[:B * I].view(B, I), self.gate_up[B * I:].view(B, I)
         x, h = self.x_res, self.h_norm
-        # With one or two rows the element-wise work rides inside the look-up kernel
-        # (five launches per block); larger batches go through the matrix-core kernel,
-        # which has no fused transforms, with the glue kernels in between (eight).
-        fold = self.fuse and B <= 2
+        # With grouped launches on, q,k,v and gate,up overwrite their outputs and, with one
+        # or two rows (look-up kernel), SiLU*up rides inside the down_proj kernel: seven
+        # launches per block, eight with more rows.  Without grouped launches the glue
+        # kernels also clear the accumulate-into outputs.
+        fold = self.fuse
+        fold_gate = fold and B <= 2                         # input transforms live in the look-up kernel
+        fold_norm = fold_gate and self.fold_norm
         torch.index_select(self.embed, 0, self.ids, out=x)
         for li, blk in enumerate(self.blocks):
             qkv_lins = [blk.q_proj, blk.k_proj, blk.v_proj]
-            if fold and self.fold_norm:
+            if fold_norm:
                 self._fused_gemv(qkv_lins, x, [q, k, v], sp, norm=blk.input_norm, overwrite=True)
             elif fold:
                 check(lib.lutgemm_decode_rmsnorm_f16(x.data_ptr(), blk.input_norm.data_ptr(), h.data_ptr(), B,
@@ -247,13 +250,17 @@ class LutDecoder(nn.Module):
                                                    self.att.data_ptr(), B, H, KV, hd, cfg.max_positions, sp))
             self._gemv_into([blk.o_proj], self.att, [x], sp)            # x += o_proj(att)
             if fold:
-                if self.fold_norm:
+                if fold_norm:
                     self._fused_gemv([blk.gate_proj, blk.up_proj], x, [g, u], sp, norm=blk.post_norm, overwrite=True)
                 else:
                     check(lib.lutgemm_decode_rmsnorm_f16(x.data_ptr(), blk.post_norm.data_ptr(), h.data_ptr(), B,
                                                          cfg.hidden, cfg.rms_eps, None, 0, sp))
                     self._fused_gemv([blk.gate_proj, blk.up_proj], h, [g, u], sp, overwrite=True)
-                self._fused_gemv([blk.down_proj], u, [x], sp, gate=g)   # x += down_proj(silu(g) * u)
+                if fold_gate:
+                    self._fused_gemv([blk.down_proj], u, [x], sp, gate=g)   # x += down_proj(silu(g) * u)
+                else:
+                    check(lib.lutgemm_decode_silu_mul_f16(g.data_ptr(), u.data_ptr(), self.act.data_ptr(), B * I, sp))
+                    self._gemv_into([blk.down_proj], self.act, [x], sp)
             else:
                 check(lib.lutgemm_decode_rmsnorm_f16(x.data_ptr(), blk.post_norm.data_ptr(), h.data_ptr(), B,
                                                      cfg.hidden, cfg.rms_eps, self.gate_up.data_ptr(),

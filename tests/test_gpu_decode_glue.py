@@ -175,7 +175,8 @@ def test_fused_rmsnorm_gemv_equals_separate_kernels(gpu_device, M, K, Ns, nbs):
         assert rel <= 2e-3 and mad <= 1e-2, (rel, mad)
 
 
-@pytest.mark.parametrize("M,K,N,nb", [(1, 11008, 4096, 3), (2, 1408, 512, 4), (4, 512, 256, 2)])
+@pytest.mark.parametrize("M,K,N,nb", [(1, 11008, 4096, 3), (2, 1408, 512, 4), (4, 512, 256, 2),
+                                        (8, 11008, 4096, 3), (33, 1024, 528, 4)])    # several rows: matrix-core kernel
 def test_fused_swiglu_gemv_equals_separate_kernels(gpu_device, M, K, N, nb):
     lib = native.cabi()
     g = torch.Generator(device=gpu_device).manual_seed(M * 13 + K)
@@ -206,3 +207,19 @@ def test_fused_entry_point_rejects_bad_problems(gpu_device):
     arr = (native.FusedProblem * 1)()
     assert lib.lutgemm_gemv_rowwise_f16_fused(0, arr, _sp()) == -1
     assert lib.lutgemm_gemv_rowwise_f16_fused(native.MAX_GROUP + 1, arr, _sp()) == -1
+
+
+@pytest.mark.parametrize("M", [1, 2, 8, 20])
+def test_overwrite_mode_ignores_previous_output(gpu_device, M):
+    lib = native.cabi()
+    g = torch.Generator(device=gpu_device).manual_seed(M)
+    x = torch.randn((M, 1024), generator=g, device=gpu_device).half()
+    lins = [_random_lin(gpu_device, N, 1024, nb, 3 * N) for N, nb in ((512, 3), (1024, 2))]
+    want = [torch.zeros((M, l[2]), dtype=torch.float16, device=gpu_device) for l in lins]
+    for l, o in zip(lins, want):
+        _plain(lib, l, x, o)
+    got = [torch.full((M, l[2]), float("nan"), dtype=torch.float16, device=gpu_device) for l in lins]
+    _ok(_fused_call(lib, lins, x, got, overwrite=True))
+    torch.cuda.synchronize()
+    for a, b in zip(got, want):
+        assert torch.allclose(a.float(), b.float(), rtol=2e-3, atol=2e-3 * float(b.float().abs().max()))
