@@ -525,3 +525,49 @@ def test_grouped_launch_rejects_overlapping_outputs(gpu_device):
     assert lib.lutgemm_gemv_rowwise_f16_grouped(2, arr, _stream()) == 0
     torch.cuda.synchronize()
     assert torch.equal(out[:, :256], out[:, 256:])
+
+
+@pytest.mark.parametrize("N,K,nb", [(28672, 8192, 4), (8192, 28672, 2)])
+def test_config5_largest_shapes_by_size_independent_properties(gpu_device, N, K, nb):
+    """The two largest 70B shapes, too big for the scalar oracle within the suite's
+    budget: exact columns for unit vectors (the dequantised entry is computed from the
+    sign bit and the alphas directly), for the look-up kernel (1 row) and the
+    matrix-core kernel (6 and 20 rows); linearity; rows of a batch against single rows."""
+    g = torch.Generator(device=gpu_device).manual_seed(N + nb)
+    bW = torch.randint(-2 ** 31, 2 ** 31 - 1, (K // 32, nb, N), generator=g, device=gpu_device, dtype=torch.int32)
+    e = torch.randint(-9, -5, (K // 128, 1, N), generator=g, device=gpu_device).float()
+    alpha = torch.exp2(e - torch.arange(nb, device=gpu_device).float().view(1, nb, 1)).half().contiguous()
+    lib = native.cabi()
+    vp = lambda t: ctypes.c_void_p(t.data_ptr())
+
+    def call(x):
+        out = torch.zeros((x.shape[0], N), dtype=torch.float16, device=gpu_device)
+        rc = lib.lutgemm_gemv_rowwise_f16(vp(bW), vp(alpha), vp(x), vp(out), N, K, nb, K // 128, x.shape[0], _stream())
+        assert rc == 0, lib.lutgemm_strerror(rc).decode()
+        torch.cuda.synchronize()
+        return out
+
+    def column(k):          # W_q[:, k] = sum_b alpha[k // 128][b] * (2 * bit - 1), exact in fp16 here
+        bits = (bW[k // 32] >> (k % 32)) & 1                          # [nb, N]
+        return ((2 * bits - 1).float() * alpha[k // 128].float()).sum(dim=0)
+
+    ks = [0, 31, 32, 127, 128, K // 2 + 5, K - 33, K - 1]
+    for rows in (1, 6, 20):
+        pick = (ks * 3)[:rows]
+        x = torch.zeros((rows, K), dtype=torch.float16, device=gpu_device)
+        for i, k in enumerate(pick):
+            x[i, k] = 1.0
+        got = call(x).float()
+        for i, k in enumerate(pick):
+            assert torch.equal(got[i], column(k)), (rows, i, k)
+    # linearity and batch/single agreement on random activations
+    x1 = torch.randn((1, K), generator=g, device=gpu_device).half()
+    x2 = torch.randn((1, K), generator=g, device=gpu_device).half()
+    y1, y2 = call(x1).float(), call(x2).float()
+    y12 = call((x1.float() + x2.float()).half()).float()
+    rel, _ = orc.error_metrics((y1 + y2).cpu().numpy(), y12.cpu().numpy())
+    assert rel < 3e-3
+    both = call(torch.cat([x1, x2, x1, x2, x1])).float()               # 5 rows: matrix-core kernel
+    for i, y in enumerate((y1, y2, y1, y2, y1)):
+        rel, _ = orc.error_metrics(both[i:i + 1].cpu().numpy(), y.cpu().numpy())
+        assert rel <= 2e-4, (i, rel)
