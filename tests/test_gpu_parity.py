@@ -571,3 +571,27 @@ def test_config5_largest_shapes_by_size_independent_properties(gpu_device, N, K,
     for i, y in enumerate((y1, y2, y1, y2, y1)):
         rel, _ = orc.error_metrics(both[i:i + 1].cpu().numpy(), y.cpu().numpy())
         assert rel <= 2e-4, (i, rel)
+
+
+@pytest.mark.parametrize("batch", [1, 8])
+def test_decoder_full_width_hip_glue_matches_framework_glue(gpu_device, batch):
+    """Two Llama-2-7B-sized blocks (hidden 4096, intermediate 11008, 32 heads of 128):
+    the fused decode step (graph replay) against the same step spelt in framework
+    operations over the same LutLinear layers, at the real shapes."""
+    from shiftaddllm_amd import decode
+    cfg = decode.DecoderConfig(vocab_size=2048, layers=2, max_positions=64)
+    qc = workload.mixed_bit_config(cfg.layers, seed=1)
+    ids = torch.randint(0, cfg.vocab_size, (batch, 5), generator=torch.Generator().manual_seed(2))
+    outs = {}
+    for glue in ("hip", "torch"):
+        model = decode.LutDecoder(cfg, qc, batch=batch, seed=7, device=gpu_device, glue=glue)
+        if glue == "hip":
+            model.capture()
+        model.reset()
+        seq = [model.forward_token(ids[:, t].to(gpu_device), t).float().cpu().clone() for t in range(ids.shape[1])]
+        torch.cuda.synchronize()
+        outs[glue] = torch.stack(seq)
+        del model
+    rel, mad = orc.error_metrics(outs["hip"].numpy().reshape(-1, cfg.vocab_size),
+                                 outs["torch"].numpy().reshape(-1, cfg.vocab_size))
+    assert rel <= 5e-3 and mad <= 2e-2, (rel, mad)       # two fp16 networks with differently rounded glue
