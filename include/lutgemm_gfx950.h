@@ -21,9 +21,24 @@
  *           (mv_fp16_bias.hpp:101,216,324,491,577; lut_gemm/quant.py:46).
  *           Unlike the reference's fp16 atomics the sum is formed in fp32 and
  *           rounded to fp16 once, and it is deterministic.
+ *           A sum that is not finite comes out as it would from IEEE
+ *           arithmetic (NaN stays NaN, +inf and -inf give NaN), whatever the
+ *           launch plan; partial sums beyond +-65536 count as infinite.
  * Shape rules enforced here (the reference checks nothing and reads or writes
- * out of bounds instead): K % 32 == 0, N % 4 == 0, 1 <= nb <= 4, M >= 1,
- * 16-byte aligned bW, 8-byte aligned row-wise alpha.
+ * out of bounds instead): K % 32 == 0, N % 4 == 0, 1 <= nb <= 4,
+ * 1 <= M <= 65535, 16-byte aligned bW and x, 8-byte aligned row-wise alpha and out.
+ *
+ * Workspace.  K is split over workgroups whose partial sums meet in one 64-bit
+ * word per output, M * N words per call, which the library keeps per (device,
+ * stream): grow-only, zero between launches.  The first call that needs more
+ * words than the stream has synchronises the stream and allocates; that cannot
+ * happen while the stream is being captured (LUTGEMM_ECAPTURE), so either make
+ * one call of each shape before capturing or reserve the words up front with
+ * lutgemm_reserve_workspace().  A captured graph names the workspace of the
+ * stream it was captured on: replay graphs captured on ONE stream one at a
+ * time (whatever stream they are replayed on), and do not run eager calls on
+ * that stream while one of its graphs is replaying -- both would share
+ * accumulator words.  Graphs captured on different streams are independent.
  */
 #ifndef LUTGEMM_GFX950_H
 #define LUTGEMM_GFX950_H
@@ -41,6 +56,8 @@ extern "C" {
 #define LUTGEMM_EUNSUP (-3)   /* legal in the reference API, not built here */
 #define LUTGEMM_EHIP (-4)     /* a HIP runtime call failed                  */
 #define LUTGEMM_ENOMEM (-5)   /* workspace allocation failed                */
+#define LUTGEMM_ECAPTURE (-6) /* the stream is being captured and its workspace
+                                 would have to grow: reserve it beforehand   */
 
 /* Human-readable text for a return code (static storage). */
 const char *lutgemm_strerror(int code);
@@ -145,6 +162,29 @@ size_t lutgemm_algorithmic_bytes(int N, int K, int nb, int M, size_t alpha_entri
  * counters against a known traffic.  No counterpart in the reference.
  */
 int lutgemm_copy_bytes(void *dst, const void *src, size_t bytes, void *stream);
+
+/*
+ * Words (8 bytes each) of accumulator workspace a call with these sizes needs at
+ * most, and a way to provide them ahead of time: after
+ * lutgemm_reserve_workspace(stream, w) no call on `stream` whose sizes need at
+ * most w words synchronises or allocates, so such calls can be captured into a
+ * HIP graph without a warm-up call.  For a grouped or fused call add up the
+ * words of its problems.  Reserving synchronises `stream` and may not be done
+ * while it is being captured (LUTGEMM_ECAPTURE).  No counterpart in the
+ * reference, whose kernels accumulate with fp16 atomics straight into `out`.
+ */
+size_t lutgemm_workspace_words(int N, int M);
+int lutgemm_reserve_workspace(void *stream, size_t words);
+
+/*
+ * Measurement helpers for the floors any kernel of this library sits on (no
+ * counterpart in the reference): a kernel that streams `bytes` (multiple of 16)
+ * from `src` with the same 128-bit non-temporal loads as the look-up kernel and
+ * does nothing with them (`sink`: 4 writable bytes, or NULL), and an empty
+ * kernel with the look-up kernel's workgroup size and LDS footprint.
+ */
+int lutgemm_measure_stream_read(const void *src, size_t bytes, void *sink, void *stream);
+int lutgemm_measure_empty_launch(int workgroups, void *stream);
 
 /* Release the per-stream workspaces this library allocated on the current
  * device (optional; they otherwise live until the process ends).  HIP graphs

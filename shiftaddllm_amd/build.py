@@ -45,25 +45,32 @@ def _run(cmd):
     subprocess.check_call(cmd)
 
 
-KERNEL_SOURCES = ("lutgemm_kernels.hip", "decode_kernels.hip")
+KERNEL_SOURCES = ("lutgemm_host.hip", "lut_gemv_rowwise.hip", "lut_gemv_block.hip", "lut_gemv_block_staged.hip",
+                  "lut_gemv_group.hip", "lut_gemm_mfma.hip", "decode_kernels.hip")
+KERNEL_HEADERS = ("lutgemm_internal.h", "lutgemm_common.h", "lutgemm_launch.h", "lut_gemv_device.h",
+                  "lut_gemm_mfma_device.h")
 
 
 def build_kernel_library(force: bool = False) -> str:
-    """One object per source (only stale ones are recompiled), linked into the library."""
-    hdrs = [os.path.join(INCLUDE, "lutgemm_gfx950.h"), os.path.join(CSRC, "lutgemm_internal.h")]
+    """One object per source (only stale ones are recompiled, several at a time), linked into the library."""
+    from concurrent.futures import ThreadPoolExecutor
+
+    hdrs = [os.path.join(INCLUDE, "lutgemm_gfx950.h")] + [os.path.join(CSRC, h) for h in KERNEL_HEADERS]
     hipcc = os.path.join(ROCM, "bin", "hipcc")
     obj_dir = os.path.join(CSRC, "build")
     os.makedirs(obj_dir, exist_ok=True)
     flags = [f for f in HIPCC_FLAGS if f != "-shared"]
-    objs, relink = [], force or not os.path.exists(KERNEL_LIB)
+    objs, stale = [], []
     for name in KERNEL_SOURCES:
         src = os.path.join(CSRC, name)
         obj = os.path.join(obj_dir, os.path.splitext(name)[0] + ".o")
         if force or not _newer(obj, src, *hdrs):
-            _run([hipcc, *flags, "-I", INCLUDE, "-c", "-o", obj, src])
-            relink = True
+            stale.append([hipcc, *flags, "-I", INCLUDE, "-I", CSRC, "-c", "-o", obj, src])
         objs.append(obj)
-    if relink or not _newer(KERNEL_LIB, *objs):
+    jobs = max(1, min(len(stale), int(os.environ.get("MAX_JOBS", "0")) or (os.cpu_count() or 4), 8))
+    with ThreadPoolExecutor(max_workers=jobs) as pool:
+        list(pool.map(_run, stale))
+    if stale or force or not _newer(KERNEL_LIB, *objs):
         _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", KERNEL_LIB, *objs])
     return KERNEL_LIB
 

@@ -1,0 +1,699 @@
+// Table look-up GEMV kernel templates for BCQ linear layers on MI355X (gfx950,
+// wave64).  One template covers the five operand formats of the reference
+// extension (lut_gemm/mv_fp16_bias.hpp:8-103,105-220,223-328,342-495,498-579 in
+// the ShiftAddLLM checkout); the operand layouts are the reference's, the
+// execution scheme is not:
+//
+//  * Work items are (N-tile of 256 outputs, "set" of 256 inputs = 8 sign words =
+//    32 eight-input chunks), numbered tile-major.  A workgroup (512 threads = 8
+//    waves) takes a contiguous range of items, so every workgroup of a launch
+//    has the same amount of work whatever the shape; a range may end one tile's
+//    K-slice and begin the next tile's.
+//  * Per item the workgroup builds 32 partial-sum tables of 256 fp32 entries in
+//    LDS.  Entry i of table t of buffer f sits at byte i*256 + 4*(t + 32*f):
+//    every table lives entirely in LDS bank t, and two buffers interleave in the
+//    same 64 KiB so that the tables of item i+1 are built while item i is looked
+//    up (one barrier per item).  A half-wave is arranged so that its 32 lanes
+//    always look up 32 different tables, hence 32 different banks: no bank
+//    conflicts by construction, whatever the data-dependent indices are.
+//  * The 256-byte entry stride makes a look-up address "index byte in bits
+//    8..15, per-lane bank offset in bits 0..7", which ONE v_perm_b32 assembles
+//    from the sign word and a per-lane constant; a look-up costs that, the
+//    ds_read_b32 and one fma.
+//  * Lane l of a wave: q = l&3, kw = (l>>2)&7, h = l>>5.  The lane streams
+//    128-bit loads of sign word (set*8 + kw) for the 4 outputs of quad
+//    (h*4+q); rows of the sign matrix are read in 1 KiB contiguous runs per
+//    workgroup.  At look-up step j the lane uses byte (j+q)&3 of its word,
+//    i.e. table kw*4 + ((j+q)&3) -- distinct over (kw, q).
+//  * Two register buffers hold the operands of items i and i+1: the loads of
+//    item i+1 are issued before the tables of item i are built and looked up,
+//    so a load has a whole item's time to arrive, and the first two items of a
+//    range are requested before anything is waited for.
+//  * Accumulation is fp32; alphas are applied with one fma per look-up (a
+//    power-of-two alpha is then an exact exponent shift).  At the end of a
+//    tile's K-slice the 8 kw-lanes of an output are combined by a reduce-scatter
+//    over ds_swizzle (4 exchanges), which leaves ONE output per lane, 32
+//    consecutive outputs per wave.
+//  * K is split over workgroups.  Each adds its partial sums, as 64-bit fixed
+//    point, into a per-output accumulator word with ONE returning atomic per
+//    lane (a wave's 32 atomics fall into two cache lines); the top byte of the
+//    word counts contributions, so the contributor that completes the count owns
+//    the sum, adds the caller's fp16 output, rounds once and clears the word.
+//    Integer addition is associative: the result does not depend on arrival
+//    order.  No fences (a device-scope release costs tens of microseconds here)
+//    and no second pass.  In "deferred" mode the atomics do not return and
+//    nobody finishes: a later kernel reads the words.
+#ifndef LUT_GEMV_DEVICE_H
+#define LUT_GEMV_DEVICE_H
+
+#include <type_traits>
+
+#include "lutgemm_common.h"
+
+namespace lutgemm {
+
+// Decode one block-alpha multiplier.
+template <int MODE>
+__device__ __forceinline__ float load_block_alpha(const void *alpha, size_t i)
+{
+    if constexpr (MODE == kBlockF16) {
+        return __half2float(((const __half *)alpha)[i]);
+    } else if constexpr (MODE == kBlockShiftU16) {
+        const uint32_t u = ((const uint16_t *)alpha)[i];
+        return (float)((1u << (u & 7u)) + (1u << ((u >> 3) & 7u)) + (1u << ((u >> 6) & 7u)));
+    } else {
+        const int8_t *s = (const int8_t *)alpha + 3 * i;
+        float a = 0.0f;
+#pragma unroll
+        for (int t = 0; t < 3; ++t) {
+            const int e = s[t];
+            a += (e == -128) ? 0.0f : ldexpf(1.0f, e);  // exponent shift, no multiplier
+        }
+        return a;
+    }
+}
+
+// Everything one lane needs from global memory for one item.
+template <int NB, int MODE>
+struct ItemOperands {
+    u32x4 w[NB];        // sign words: 4 outputs x 32 inputs per register quad
+    u32x2 a_row[NB];    // row-wise: 4 fp16 alphas (one per output)
+    float a_blk[NB][4]; // block: one multiplier per look-up step
+    u32x2 a_uni;        // uniform: alpha per output
+    u32x2 q_uni;        // uniform: q_bias per output
+    float a_stage;      // staged block modes: the one alpha this thread stages
+    int rgroup;         // staged block modes: alpha row group of the lane's quad, relative to the tile's first
+};
+
+// Issue every global load of item (tile, set) for this lane.  Branch-free on
+// purpose: out-of-range rows and columns are clamped to valid addresses instead
+// of predicated, so the loads sit in straight-line code and the compiler can
+// keep later items' loads in flight (s_waitcnt vmcnt(n), n > 0) while the
+// current item is consumed.  Clamped data is harmless: tables of inputs beyond K
+// are all zero, and outputs beyond N are never written.  An item that does not
+// exist (`valid` false, the slot after the last item of a range) is "loaded" too,
+// with every lane pointed at the first words of the operands: a handful of cache
+// lines instead of a conditional load.  Addresses are a uniform 64-bit base plus a
+// 32-bit per-lane offset.
+template <int NB, int MODE>
+__device__ __forceinline__ void load_item(ItemOperands<NB, MODE> &r, const Problem &p, int tile, int set, bool valid,
+                                          int kw, int q, int lane_col, int tid)
+{
+    tile = valid ? tile : 0;
+    set = valid ? set : 0;
+    const uint32_t lane_mask = valid ? ~0u : 0u;
+    const int tile0 = tile * kTileCols;
+    const int n = min(tile0 + lane_col, p.N - 4);
+    const uint32_t col4 = (uint32_t)n * 4u, col2 = (uint32_t)n * 2u;
+    const int kwc = min(kw, p.kwords - 1 - set * kSetWords);  // only the last set of K can clamp
+    const uint32_t row_bytes = (uint32_t)p.N * 4u;            // one bit plane of one sign word row
+    const char *wbase = (const char *)p.W + (size_t)set * kSetWords * NB * row_bytes;
+    const uint32_t wrow = (uint32_t)kwc * (NB * row_bytes);
+    [[maybe_unused]] const int row = set * kSetWords + kwc;
+    [[maybe_unused]] const int g = fast_div(row, p.by_group_words);  // alpha group of the row
+    const uint32_t woff = (wrow + col4) & lane_mask;
+#pragma unroll
+    for (int b = 0; b < NB; ++b) {
+        const char *src = wbase + (size_t)b * row_bytes;
+        r.w[b] = __builtin_nontemporal_load((const u32x4 *)(src + woff));
+    }
+    if constexpr (MODE == kRowF16) {
+        const uint32_t aoff = ((uint32_t)g * (NB * (uint32_t)p.N * 2u) + col2) & lane_mask;
+#pragma unroll
+        for (int b = 0; b < NB; ++b) {
+            const char *src = (const char *)p.alpha + (size_t)b * p.N * 2u;
+            r.a_row[b] = *(const u32x2 *)(src + aoff);
+        }
+    } else if constexpr (MODE == kUniformF16) {
+        const uint32_t aoff = ((uint32_t)g * ((uint32_t)p.N * 2u) + col2) & lane_mask;
+        r.a_uni = *(const u32x2 *)((const char *)p.alpha + aoff);
+        r.q_uni = *(const u32x2 *)((const char *)p.qbias + aoff);
+    } else if constexpr (is_block(MODE)) {
+        const int rgroup = n / p.rows_per_group;
+#pragma unroll
+        for (int b = 0; b < NB; ++b)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int chunk = row * 4 + ((j + q) & 3);
+                r.a_blk[b][j] = load_block_alpha<MODE>(p.alpha, ((size_t)chunk * NB + b) * p.R + rgroup);
+            }
+    }
+    if constexpr (is_staged(MODE)) {
+        // thread t stages alpha(chunk c of the set, bit b, row group rg0 + g2)
+        const int rg0 = tile0 / p.rows_per_group;
+        r.rgroup = n / p.rows_per_group - rg0;
+        const int t = tid % (2 * NB * kTables);
+        const int c = t % kTables, b = (t / kTables) % NB, g2 = t / (NB * kTables);
+        const int chunk = min(set * kTables + c, p.K / 8 - 1);
+        const int rg = min(rg0 + g2, p.R - 1);
+        r.a_stage = load_block_alpha<base_mode(MODE)>(p.alpha, ((size_t)chunk * NB + b) * p.R + rg);
+    }
+}
+
+// Staged block modes: publish this thread's alpha of an item into stage buffer `abuf`.
+template <int NB, int MODE>
+__device__ __forceinline__ void stage_alpha(const ItemOperands<NB, MODE> &ops, float *stage, int abuf, int tid)
+{
+    if constexpr (is_staged(MODE)) {
+        if (tid < 2 * NB * kTables) {
+            const int c = tid % kTables, b = (tid / kTables) % NB, g2 = tid / (NB * kTables);
+            stage[((abuf * 2 + g2) * 4 + b) * kTables + c] = ops.a_stage;
+        }
+    }
+}
+
+// Activation window.  The activations a workgroup needs are few (512 bytes per item
+// and row), so they are not fetched item by item: thread t of the workgroup loads ONE
+// 16-byte chunk (8 inputs) of a window of kWindowSlots/MROWS consecutive items, applies
+// the fused input transform to it once, and parks it in LDS, where the table builds
+// read it.  The builds then wait for no global load at all, and the loads that stream
+// sign words are the only ones in the (in-order) return queue of the steady state.
+// Window layout: [row][slot = item index within the range, modulo slots per row][chunk].
+constexpr int kWindowSlots = kThreads / kTables;       // 16 (item, row) slots of 32 chunks
+constexpr int kWindowDwords = kWindowSlots * kTables * 4;  // 8 KiB
+
+// What thread `tid` fetches for the window that starts `first_rel` items into the range.
+struct WindowChunk {
+    u32x4 x, other;
+    int kc;     // first input of the chunk (clamped into the row)
+    bool live;  // chunks beyond K, or of items beyond the range, read as zero
+};
+
+template <int MROWS, int XF>
+__device__ __forceinline__ WindowChunk fetch_window(const Problem &p, int m0, int set0, int first_rel, int n_items,
+                                                    int tid)
+{
+    constexpr int kSlots = kWindowSlots / MROWS;  // items per window
+    const int c = tid % kTables, slot = (tid / kTables) % kSlots, row = tid / (kTables * kSlots);
+    const int rel = first_rel + slot;
+    const int v = set0 + rel;
+    const int set = v - fast_div(v, p.by_nsets) * p.nsets;
+    const int k0 = (set * kTables + c) * 8;
+    const int kc = min(k0, p.K - 8);
+    const size_t base = (size_t)min(m0 + row, p.M - 1) * p.K + kc;
+    WindowChunk w;
+    w.x = *(const u32x4 *)(p.x + base);
+    w.other = (u32x4){0u, 0u, 0u, 0u};
+    // (the norm weight is read when the chunk is finished: a few KB shared by all
+    // workgroups, and four registers less are held until then)
+    if constexpr (XF == kXGate) w.other = *(const u32x4 *)(p.gate + base);
+    w.kc = kc;
+    w.live = k0 < p.K && rel < n_items;
+    return w;
+}
+
+// Transform the chunk and park it in the window.  With a norm weight the chunk is
+// scaled by the row's reciprocal RMS and the weight; with a gate row it is multiplied
+// by silu(gate); both with the roundings of the separate fp16 operations they replace.
+template <int MROWS, int XF>
+__device__ __forceinline__ void store_window(const Problem &p, const WindowChunk &w, const float (&rscale)[MROWS],
+                                             float *window, int tid)
+{
+    u32x4 xr = w.x;
+    // (opaque: the work on the fetched chunk stays here, after the sign-word requests,
+    // instead of being hoisted to where it would have to wait for the chunk first)
+    asm volatile("" : "+v"(xr.x), "+v"(xr.y), "+v"(xr.z), "+v"(xr.w));
+    if constexpr (XF != kXNone) {
+        constexpr int kSlots = kWindowSlots / MROWS;
+        const int row = tid / (kTables * kSlots);
+        float rs = rscale[0];
+#pragma unroll
+        for (int r = 1; r < MROWS; ++r) rs = row == r ? rscale[r] : rs;
+        u32x4 other = w.other;
+        if constexpr (XF == kXNorm) other = *(const u32x4 *)(p.norm_w + w.kc);
+        const uint32_t a[4] = {xr.x, xr.y, xr.z, xr.w};
+        const uint32_t b[4] = {other.x, other.y, other.z, other.w};
+        uint32_t o[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            float v[2];
+#pragma unroll
+            for (int hh = 0; hh < 2; ++hh) {
+                const float xv = half_bits_to_float((a[j] >> (16 * hh)) & 0xffffu);
+                const float bv = half_bits_to_float((b[j] >> (16 * hh)) & 0xffffu);
+                if constexpr (XF == kXGate)
+                    v[hh] = half_bits_to_float(float_to_half_bits(__fdividef(bv, 1.0f + __expf(-bv)))) * xv;
+                else
+                    v[hh] = half_bits_to_float(float_to_half_bits(xv * rs)) * bv;
+            }
+            o[j] = float_to_half_bits(v[0]) | (float_to_half_bits(v[1]) << 16);
+        }
+        xr = (u32x4){o[0], o[1], o[2], o[3]};
+    }
+    u32x4 r;
+    r.x = w.live ? xr.x : 0u;
+    r.y = w.live ? xr.y : 0u;
+    r.z = w.live ? xr.z : 0u;
+    r.w = w.live ? xr.w : 0u;
+    *(u32x4 *)(window + 4 * tid) = r;
+}
+
+// Build the 32 tables of one item into buffer `buf` (0/1).  Thread (tb, eb)
+// writes entries eb*16 .. eb*16+15 of table tb: bits 4..7 of the entry index
+// come from eb, bits 0..3 are walked in Gray-code order, one add per entry.
+__device__ __forceinline__ void build_tables(const u32x4 &xraw, float *lut, int buf, int tb, int eb)
+{
+    float x2[8];  // 2 * x
+    float base = 0.0f;
+    const uint32_t r4[4] = {xraw.x, xraw.y, xraw.z, xraw.w};
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const float lo = half_bits_to_float(r4[j] & 0xffffu);
+        const float hi = half_bits_to_float(r4[j] >> 16);
+        x2[2 * j] = lo + lo;
+        x2[2 * j + 1] = hi + hi;
+        base -= lo + hi;  // entry 0 = -sum x
+    }
+    float top = base;
+#pragma unroll
+    for (int j = 4; j < 8; ++j)
+        if ((eb >> (j - 4)) & 1) top += x2[j];
+    float *col = lut + (eb * 16) * kEntryStride + buf * kTables + tb;
+#pragma unroll
+    for (int sb = 0; sb < 2; ++sb) {  // bit 3 fixed per sub-block: two short chains
+        float v = top;
+        if (sb & 1) v += x2[3];
+        unsigned gray = 0;
+        col[(sb * 8) * kEntryStride] = v;
+#pragma unroll
+        for (int i = 1; i < 8; ++i) {
+            const int bit = __builtin_ctz(i);
+            gray ^= 1u << bit;
+            v += ((gray >> bit) & 1u) ? x2[bit] : -x2[bit];
+            col[(sb * 8 + gray) * kEntryStride] = v;
+        }
+    }
+}
+
+// This lane's look-ups of one item against the table buffer `lane_off` selects.
+// lane_off: byte j = 4*(bank of the table used at step j + 32*buffer).
+// sel[j]  : v_perm_b32 selector putting byte (j+q)&3 of the sign word into
+//           bits 8..15 and byte j of lane_off into bits 0..7.
+// Software pipelined in units of 8 look-ups (one bit plane of two outputs): the LDS
+// reads of unit u+1 are issued before the fmas of unit u.  (Units of 16 cost 16 more
+// registers, which four bit planes do not have to spare.)
+template <int NB, int MODE>
+__device__ __forceinline__ void lookup_item(const ItemOperands<NB, MODE> &cur, const float *lut, float (&acc)[4],
+                                            uint32_t lane_off, const uint32_t (&sel)[4], const float *stage_lane,
+                                            int q)
+{
+    const char *lut_bytes = (const char *)lut;
+    constexpr int kUnits = 2 * NB;   // a unit = 8 look-ups: one bit plane of two outputs
+    float val[2][8];
+    [[maybe_unused]] float aval[2][4];
+    auto issue = [&](int u, float (&v)[8], float (&av)[4]) {
+        const int b = u >> 1, i0 = (u & 1) * 2;
+        const uint32_t w4[4] = {cur.w[b].x, cur.w[b].y, cur.w[b].z, cur.w[b].w};
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                v[4 * i + j] = *(const float *)(lut_bytes + __builtin_amdgcn_perm(w4[i0 + i], lane_off, sel[j]));
+        if constexpr (is_staged(MODE)) {
+            // stage_lane points at [this item's buffer][group 0][bit 0][kw*4]; the four
+            // alphas of the lane's sign word, in look-up step order
+            const float *a4 = stage_lane + (cur.rgroup * 4 + b) * kTables;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) av[j] = a4[(j + q) & 3];
+        }
+    };
+    auto retire = [&](int u, const float (&v)[8], const float (&av)[4]) {
+        const int b = u >> 1, i0 = (u & 1) * 2;
+        [[maybe_unused]] const uint32_t ar = (u & 1) ? cur.a_row[b].y : cur.a_row[b].x;
+        [[maybe_unused]] const uint32_t au = (u & 1) ? cur.a_uni.y : cur.a_uni.x;
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            float a = 0.0f;
+            if constexpr (MODE == kRowF16)
+                a = half_bits_to_float((ar >> (16 * i)) & 0xffffu);
+            else if constexpr (MODE == kUniformF16)
+                a = half_bits_to_float((au >> (16 * i)) & 0xffffu) * (1.0f / (float)(2 << b));
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                if constexpr (is_block(MODE))
+                    a = cur.a_blk[b][j];
+                else if constexpr (is_staged(MODE))
+                    a = av[j];
+                acc[i0 + i] = fmaf(v[4 * i + j], a, acc[i0 + i]);
+            }
+        }
+    };
+    issue(0, val[0], aval[0]);
+    if constexpr (MODE == kUniformF16) {
+        // sum of the lane's 32 inputs = entry 255 of its four tables
+        float sum_x = 0.0f;
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+            sum_x += *(const float *)(lut_bytes + 255 * 4 * kEntryStride + ((lane_off >> (8 * j)) & 255u));
+        const uint32_t rq[2] = {cur.q_uni.x, cur.q_uni.y};
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            acc[i] = fmaf(half_bits_to_float((rq[i >> 1] >> (16 * (i & 1))) & 0xffffu), sum_x, acc[i]);
+    }
+#pragma unroll
+    for (int u = 0; u < kUnits; ++u) {
+        if (u + 1 < kUnits) issue(u + 1, val[(u + 1) & 1], aval[(u + 1) & 1]);
+        retire(u, val[u & 1], aval[u & 1]);
+    }
+}
+
+// ds_swizzle in bit-mask mode: the value of lane (l ^ XOR) within each group of 32.
+template <int XOR>
+__device__ __forceinline__ float swizzle_xor(float v)
+{
+    return __builtin_bit_cast(float, __builtin_amdgcn_ds_swizzle(__builtin_bit_cast(int, v), (XOR << 10) | 0x1f));
+}
+
+// Reduce-scatter of the 8 kw-lanes of a quad: each lane comes in with its partial
+// sums of 4 outputs and leaves with the complete sum of output
+// i = 2*(kw>>2 & 1) + (kw>>1 & 1); lanes kw and kw^1 hold the same value.
+__device__ __forceinline__ float reduce_scatter_kw(const float (&acc)[4], int kw)
+{
+    const bool b2 = (kw >> 2) & 1, b1 = (kw >> 1) & 1;
+    float k0 = b2 ? acc[2] : acc[0], k1 = b2 ? acc[3] : acc[1];   // kept
+    const float s0 = b2 ? acc[0] : acc[2], s1 = b2 ? acc[1] : acc[3];  // sent to lane ^ 16
+    k0 += swizzle_xor<16>(s0);
+    k1 += swizzle_xor<16>(s1);
+    float k = b1 ? k1 : k0;
+    const float s = b1 ? k0 : k1;
+    k += swizzle_xor<8>(s);
+    k += swizzle_xor<4>(k);
+    return k;
+}
+
+// One workgroup's share: items [range*items_per_wg, +items_per_wg) of row chunk
+// `mchunk` (activation rows mchunk*MROWS .. +MROWS-1).  The sign words of an item
+// are loaded once and used for all MROWS rows; tables are built per (item, row)
+// and double buffered.
+template <int NB, int MODE, int MROWS, int XF = kXNone>
+__device__ __forceinline__ void gemv_range(const Problem &p, int range, int mchunk, float *lut)
+{
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int q = lane & 3;
+    const int kw = (lane >> 2) & 7;
+    const int h = lane >> 5;
+    const int lane_col = wave * kWaveCols + (h * 4 + q) * 4;  // first of the lane's 4 outputs within a tile
+    const int m0 = mchunk * MROWS;
+    // The output this lane owns after the reduce-scatter: own_col(kw2) with kw2 = kw.  (A
+    // function of the caller's copy of kw so that uses late in the kernel can pass an
+    // opaque copy and keep their setup out of the start-up path.)
+    auto own_col_of = [&](int kw2) { return lane_col + 2 * ((kw2 >> 2) & 1) + ((kw2 >> 1) & 1); };
+
+    // rows beyond M are clamped to the last row (computed twice, written once)
+    const __half *xrow[MROWS];
+#pragma unroll
+    for (int r = 0; r < MROWS; ++r) xrow[r] = p.x + (size_t)min(m0 + r, p.M - 1) * p.K;
+
+    // Per-lane look-up constants (see lookup_item).  Like everything else that the first
+    // requests do not depend on, they are formed after those requests have been issued
+    // (late_setup below): a workgroup's waves share their SIMDs' issue slots, and each
+    // hundred instructions ahead of the first load are a third of a microsecond.
+    uint32_t lane_off = 0;
+    uint32_t sel[4] = {0u, 0u, 0u, 0u};
+
+    float acc[MROWS][4];
+#pragma unroll
+    for (int r = 0; r < MROWS; ++r)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) acc[r][i] = 0.0f;
+
+    // table-build role of this thread
+    const int tb = tid & 31;  // table (bank)
+    const int eb = tid >> 5;  // entries eb*16 .. eb*16+15
+
+    // this workgroup's items; (tile, set) is the current one
+    const int total = p.n_tiles * p.nsets;
+    const int item0 = range * p.items_per_wg;
+    int rem = min(p.items_per_wg, total - item0);
+    int tile = fast_div(item0, p.by_nsets), set = item0 - tile * p.nsets;
+    auto advance = [&](int &t, int &s) {
+        if (++s == p.nsets) {
+            s = 0;
+            ++t;
+        }
+    };
+
+    float *stage = lut + kLutDwords;
+    int abuf = 0;
+
+    // The first activation window is requested before anything else.
+    constexpr int kSlots = kWindowSlots / MROWS;  // items per window
+    const int set0 = set, n_items = rem;
+    float *window = stage + kStageDwords;
+    const WindowChunk w0 = fetch_window<MROWS, XF>(p, m0, set0, 0, n_items, tid);
+    // Without an input transform the tables of the first item (row 0) are built straight
+    // from a second request for this thread's own chunk, so that nothing but that chunk
+    // stands between the start of the kernel and the first table.
+    u32x4 x0 = (u32x4){0u, 0u, 0u, 0u};
+    if constexpr (XF == kXNone) {
+        const int k0 = (set0 * kTables + tb) * 8;
+        x0 = *(const u32x4 *)(xrow[0] + min(k0, p.K - 8));
+    }
+
+    // fused RMSNorm: every workgroup forms the reciprocal RMS of its rows itself (K
+    // fp16 values per row, from L2), requested right behind the window.
+    constexpr int kNormChunks = 2;  // 16-byte chunks per thread held in registers: K <= 8192
+    u32x4 nx[XF == kXNorm ? MROWS : 1][kNormChunks];
+    if constexpr (XF == kXNorm) {
+#pragma unroll
+        for (int r = 0; r < MROWS; ++r)
+#pragma unroll
+            for (int u = 0; u < kNormChunks; ++u)
+                nx[r][u] = *(const u32x4 *)(xrow[r] + 8 * min(tid + kThreads * u, p.K / 8 - 1));
+    }
+    // the caller's output, needed only by whoever completes a sum: fetched early,
+    // off the critical path (again whenever the range moves on to another tile)
+    unsigned short out_prev[MROWS];
+    auto fetch_out = [&](int t) {
+        const int n = min(t * kTileCols + own_col_of(kw), p.N - 1);
+#pragma unroll
+        for (int r = 0; r < MROWS; ++r)
+            out_prev[r] = *((const unsigned short *)(p.out + (size_t)min(m0 + r, p.M - 1) * p.N) + n);
+    };
+    __builtin_amdgcn_sched_barrier(0);  // keep these requests ahead of the sign words
+
+    float rscale[MROWS];
+#pragma unroll
+    for (int r = 0; r < MROWS; ++r) rscale[r] = 1.0f;
+    // Runs once, after the first operand loads have been issued: everything the look-ups
+    // and the hand-over need but the first requests did not.
+    auto late_setup = [&]() {
+        int t = tid;
+        asm volatile("" : "+v"(t));  // (opaque, so that none of this is hoisted ahead of the requests)
+        const int lq = t & 3, lkw = (t >> 2) & 7;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int jj = (j + lq) & 3;
+            lane_off |= (uint32_t)(4 * (lkw * 4 + jj)) << (8 * j);
+            sel[j] = 0x0c0c0000u | ((uint32_t)(4 + jj) << 8) | (uint32_t)j;
+        }
+        fetch_out(tile);
+    };
+    // Also once, after that: finish the reciprocal RMS and park the first window.
+    auto first_window = [&]() {
+        if constexpr (XF == kXNorm) {
+            float ss[MROWS];
+#pragma unroll
+            for (int r = 0; r < MROWS; ++r) {
+                ss[r] = 0.0f;
+                auto add_chunk = [&](const u32x4 &v) {
+                    const uint32_t w4[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        const float lo = half_bits_to_float(w4[j] & 0xffffu), hi = half_bits_to_float(w4[j] >> 16);
+                        ss[r] = fmaf(lo, lo, fmaf(hi, hi, ss[r]));
+                    }
+                };
+#pragma unroll
+                for (int u = 0; u < kNormChunks; ++u)
+                    if (tid + kThreads * u < p.K / 8) add_chunk(nx[r][u]);
+                for (int c = tid + kThreads * kNormChunks; c < p.K / 8; c += kThreads)  // K > 16384
+                    add_chunk(*(const u32x4 *)(xrow[r] + 8 * c));
+#pragma unroll
+                for (int off = 32; off > 0; off >>= 1) ss[r] += __shfl_xor(ss[r], off);
+                if (lane == 0) lut[wave * MROWS + r] = ss[r];
+            }
+            __syncthreads();
+#pragma unroll
+            for (int r = 0; r < MROWS; ++r) {
+                float t = 0.0f;
+#pragma unroll
+                for (int w = 0; w < kWaves; ++w) t += lut[w * MROWS + r];
+                rscale[r] = rsqrtf(t / (float)p.K + p.norm_eps);
+            }
+            // (the tables are built over the same LDS words: the barrier below orders that)
+        }
+        store_window<MROWS, XF>(p, w0, rscale, window, tid);
+        // (without a transform the first build does not read the window, and the barrier
+        // that follows that build publishes the window as well)
+        if constexpr (XF != kXNone) __syncthreads();
+    };
+
+    // ---- hand a tile's complete K-slice over ---------------------------------------
+    auto flush_tile = [&](int t) {
+        // contributions this tile receives: the ranges that overlap its items
+        const int first = fast_div(t * p.nsets, p.by_items);
+        const int last = fast_div(t * p.nsets + p.nsets - 1, p.by_items);
+        const int count = last - first + 1;
+        int kw2 = kw;
+        asm volatile("" : "+v"(kw2));  // (opaque: see own_col_of)
+        const int n = t * kTileCols + own_col_of(kw2);
+        const bool owner = (kw2 & 1) == 0;
+#pragma unroll
+        for (int r = 0; r < MROWS; ++r) {
+            const float v = reduce_scatter_kw(acc[r], kw2);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) acc[r][i] = 0.0f;
+            const int m = m0 + r;
+            if (!owner || n >= p.N || m >= p.M) continue;
+            __half *dst = p.out + (size_t)m * p.N + n;
+            const float prev = p.overwrite ? 0.0f : half_bits_to_float(out_prev[r]);
+            if (count == 1 && p.finish == kFinishInline) {
+                *dst = __float2half_rn(prev + v);
+                continue;
+            }
+            unsigned long long *word = p.accum + (size_t)m * p.N + n;
+            const Contribution c = fixed_contribution(v);
+            if (c.flags) __hip_atomic_fetch_or(word, c.flags, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if (p.finish == kFinishDefer) {
+                __hip_atomic_fetch_add(word, c.add, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                continue;
+            }
+            const unsigned long long old =
+                __hip_atomic_fetch_add(word, c.add, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if ((int)(old >> 56) != count - 1) continue;
+            // this contribution completed the sum
+            *dst = __float2half_rn(prev + fixed_total((old | c.flags) + c.add, count));
+            __hip_atomic_store(word, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+    };
+
+    // Pipeline step for one item whose operands `ops` were requested earlier: per row,
+    // build the row's tables into buffer f, barrier, look them up.  The barrier both
+    // publishes buffer f and retires the readers of buffer f^1, which the next build
+    // overwrites.
+    constexpr uint32_t kFlip = 0x80808080u;  // +128 bytes = the other table buffer
+    int buf = 0;
+    int rel = 0;  // items of the range done so far
+    auto item_step = [&](const ItemOperands<NB, MODE> &ops, bool last) {
+        int nt = tile, ns = set;
+        advance(nt, ns);
+        const int slot = rel % kSlots;
+        if (rel > 0 && slot == 0) {
+            // The window is used up (every thread has passed the barrier that followed its
+            // last read): fetch and park the next one.  Not prefetched: ranges of more than
+            // a window's items only occur beyond half a billion weights per call, and a
+            // conditional load in flight would make every later wait conservative.
+            const WindowChunk w = fetch_window<MROWS, XF>(p, m0, set0, rel, n_items, tid);
+            store_window<MROWS, XF>(p, w, rscale, window, tid);
+            __syncthreads();
+        }
+#pragma unroll
+        for (int r = 0; r < MROWS; ++r) {
+            u32x4 xr = x0;
+            if (XF != kXNone || r > 0 || rel > 0) {
+                xr = *(const u32x4 *)(window + 4 * ((r * kSlots + slot) * kTables + tb));
+            } else {
+                // (opaque, so that the chunk is not waited for before it is needed)
+                asm volatile("" : "+v"(xr.x), "+v"(xr.y), "+v"(xr.z), "+v"(xr.w));
+                if ((set0 * kTables + tb) * 8 >= p.K) xr = (u32x4){0u, 0u, 0u, 0u};  // inputs beyond K
+            }
+            build_tables(xr, lut, buf, tb, eb);
+            if (r == 0) stage_alpha<NB, MODE>(ops, stage, abuf, tid);
+            __syncthreads();
+            // opaque to the optimiser: otherwise the look-up addresses of an item are
+            // kept in registers across all rows instead of being recomputed (1 op each)
+            asm volatile("" : "+v"(lane_off));
+            lookup_item<NB, MODE>(ops, lut, acc[r], lane_off, sel, stage + abuf * (2 * 4 * kTables) + kw * 4, q);
+            buf ^= 1;
+            lane_off ^= kFlip;
+        }
+        abuf ^= 1;
+        ++rel;
+        if (last || nt != tile) {
+            flush_tile(tile);
+            if (!last) fetch_out(nt);
+        }
+        tile = nt;
+        set = ns;
+    };
+    // Two operand buffers alternate: while one item is processed the next one's loads
+    // are in flight, and the first two items of the range are requested before anything
+    // is waited for.  Items are taken in pairs by a counted loop with ONE exit and ONE
+    // load site per buffer:
+    //  * with a second load site (a prologue, say) the register allocator gives the two
+    //    sites different registers and reconciles them with copies that wait for the loads;
+    //  * with a second exit the loop is restructured with edges that are never taken but
+    //    on which loads are still pending, and every iteration then starts by waiting
+    //    for everything in flight.
+    // Hence the first iteration skips its first step at run time, and the second item of
+    // the last pair, if the range has an odd number of items, is a dummy (see load_item).
+    ItemOperands<NB, MODE> opA, opB;
+    int ld_tile = tile, ld_set = set;  // next item to request
+    const int pairs = (n_items + 1) / 2;
+#pragma clang loop unroll(disable)
+    for (int j = 0; j < pairs; ++j) {
+        // (opaque, which keeps the compiler from peeling the first iteration)
+        int first = __builtin_amdgcn_readfirstlane(j == 0);
+        asm volatile("" : "+s"(first));
+        load_item<NB, MODE>(opA, p, ld_tile, ld_set, true, kw, q, lane_col, tid);
+        advance(ld_tile, ld_set);
+        if (!first) item_step(opB, false);
+        const bool has_b = 2 * j + 1 < n_items;
+        load_item<NB, MODE>(opB, p, ld_tile, ld_set, has_b, kw, q, lane_col, tid);
+        advance(ld_tile, ld_set);
+        if (first) {
+            late_setup();
+            first_window();
+        }
+        item_step(opA, !has_b);
+    }
+    if ((n_items & 1) == 0) item_step(opB, true);
+}
+
+// Flat workgroup index (relative to the problem) -> (range, row chunk), for launches
+// that hold several problems.
+__device__ __forceinline__ void decode_block(const Problem &p, int local, int &range, int &mchunk)
+{
+    mchunk = p.mchunks == 1 ? 0 : local / p.wgs_per_chunk;
+    range = local - mchunk * p.wgs_per_chunk;
+}
+
+// (at most 128 registers, so that two workgroups share a CU)
+template <int NB, int MODE, int MROWS>
+__global__ void __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4, 4)))
+lut_gemv_kernel(const Problem p)
+{
+    __shared__ __attribute__((aligned(16))) float lut[kLutDwords + kStageDwords + kWindowDwords];
+    gemv_range<NB, MODE, MROWS>(p, (int)blockIdx.x, (int)blockIdx.y, lut);  // grid = (ranges, row chunks)
+}
+
+// Several row-wise problems in one launch (flat 1-D grid).  Bit widths may
+// differ between the problems of a group.
+// XF: the input transform shared by all problems of the launch.
+template <int XF>
+__global__ void __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4, 4)))
+lut_gemv_group_kernel(const Group g)
+{
+    __shared__ __attribute__((aligned(16))) float lut[kLutDwords + kStageDwords + kWindowDwords];
+    const int b = blockIdx.x;
+    int pi = 0;
+#pragma unroll
+    for (int i = 1; i < kMaxGroup; ++i)
+        if (i < g.count && b >= g.p[i].block_begin) pi = i;
+    const Problem &p = g.p[pi];
+    int range, m;
+    decode_block(p, b - p.block_begin, range, m);
+    switch (p.nb) {
+    case 1: gemv_range<1, kRowF16, 1, XF>(p, range, m, lut); break;
+    case 2: gemv_range<2, kRowF16, 1, XF>(p, range, m, lut); break;
+    case 3: gemv_range<3, kRowF16, 1, XF>(p, range, m, lut); break;
+    default: gemv_range<4, kRowF16, 1, XF>(p, range, m, lut); break;
+    }
+}
+
+}  // namespace lutgemm
+
+#endif

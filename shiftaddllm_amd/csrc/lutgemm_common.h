@@ -1,0 +1,192 @@
+// Types and constants shared by the device templates and the host side of
+// liblutgemm_gfx950.so.  Not installed; gfx950 (wave64) only.
+#ifndef LUTGEMM_COMMON_H
+#define LUTGEMM_COMMON_H
+
+#include <hip/hip_runtime.h>
+#include <hip/hip_fp16.h>
+#include <stdint.h>
+
+#include "lutgemm_gfx950.h"
+
+namespace lutgemm {
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+constexpr int kThreads = 512;
+constexpr int kWaves = kThreads / 64;
+constexpr int kSetWords = 8;               // sign words (of 32 inputs) per table set
+constexpr int kTables = 4 * kSetWords;     // 32 tables, one per LDS bank
+constexpr int kWaveCols = 32;              // outputs a wave covers
+constexpr int kTileCols = kWaves * kWaveCols;  // outputs a workgroup covers (256)
+constexpr int kEntryStride = 64;           // dwords between consecutive entries of a table
+constexpr int kLutDwords = 256 * kEntryStride;  // 64 KiB: two interleaved table buffers
+constexpr int kStageDwords = 2 * 2 * 4 * kTables;  // staged block alphas: [buffer][row group][bit][chunk]
+constexpr int kMaxContrib = 32;            // contributions per accumulator word (see below)
+constexpr int kMaxGroup = LUTGEMM_MAX_GROUP;  // problems per grouped launch
+
+// Fixed-point accumulator word of one output (K split over workgroups):
+//   [63:56] contributions so far
+//   [55]    a contribution was -inf, below -2^16, or NaN
+//   [54]    a contribution was +inf, above +2^16, or NaN
+//   [53:0]  sum of (v + kBias), v = partial * 2^31 rounded, |partial| <= 2^16
+// kMaxContrib contributions of at most 2^48 + 2^47 stay below 2^54.  Integer
+// addition is associative, so the total does not depend on the arrival order.
+// The two flags are set with an atomic OR that precedes the contributor's add
+// (same lane, same address: performed in program order), so they are sticky and
+// every later reader of the word sees them.
+constexpr unsigned long long kCountOne = 1ull << 56;
+constexpr unsigned long long kFlagNeg = 1ull << 55;
+constexpr unsigned long long kFlagPos = 1ull << 54;
+constexpr unsigned long long kSumMask = kFlagPos - 1;
+constexpr long long kBias = 1ll << 48;
+constexpr double kFixedScale = 2147483648.0;  // 2^31
+constexpr float kFixedScaleF = 2147483648.0f;
+
+enum AlphaMode : int {
+    kRowF16 = 0,      // fp16 [G][nb][N]
+    kBlockF16 = 1,    // fp16 [K/8][nb][R]
+    kBlockShiftU16 = 2,
+    kBlockApotI8 = 3,
+    kUniformF16 = 4,  // alpha, q_bias fp16 [G][N]
+    // block formats when an N-tile spans at most two alpha row groups: the set's
+    // alphas are staged in LDS by the workgroup instead of loaded lane by lane
+    kBlockF16Staged = 5,
+    kBlockShiftU16Staged = 6,
+    kBlockApotI8Staged = 7,
+};
+
+constexpr bool is_block(int mode) { return mode == kBlockF16 || mode == kBlockShiftU16 || mode == kBlockApotI8; }
+constexpr bool is_staged(int mode) { return mode >= kBlockF16Staged; }
+constexpr int base_mode(int mode) { return is_staged(mode) ? mode - 4 : mode; }
+
+// compile-time input transform of a kernel instance
+constexpr int kXNone = 0, kXNorm = 1, kXGate = 2;
+
+// how a workgroup hands over its partial sums (Problem::finish)
+constexpr int kFinishInline = 0;  // returning atomics; the last contributor rounds and writes `out`
+constexpr int kFinishDefer = 1;   // non-returning atomics; a later kernel reads and clears the words
+
+// Division by a run-time constant without a divide: n / d == umulhi((2 * n) >> shift,
+// magic), with the pair prepared on the host (kernels here start and end within a
+// few microseconds; a software division is some thirty instructions on that path).
+// d = 2^t * o (o odd): for o == 1 the pair is (t, 2^31 + 1), i.e. (2n >> t) / 2;
+// otherwise (t + 1, floor(2^32 / o) + 1), i.e. (n >> t) / o.  The multiply-high is
+// exact while 2 * n * d < 2^32, which the host checks for every divisor it hands over.
+struct Divisor {
+    int shift;
+    uint32_t magic;
+};
+
+inline Divisor make_divisor(int d_in)
+{
+    int t = 0;
+    unsigned d = (unsigned)d_in;
+    while ((d & 1u) == 0) {
+        d >>= 1;
+        ++t;
+    }
+    Divisor r;
+    if (d == 1) {
+        r.shift = t;
+        r.magic = 0x80000001u;
+    } else {
+        r.shift = t + 1;
+        r.magic = (uint32_t)((1ull << 32) / d) + 1u;
+    }
+    return r;
+}
+
+__device__ __forceinline__ int fast_div(int n, const Divisor &d)
+{
+    return (int)__umulhi((uint32_t)(2 * n) >> d.shift, d.magic);
+}
+
+struct Problem {
+    const uint32_t *W;
+    const void *alpha;
+    const __half *qbias;
+    const __half *x;
+    __half *out;
+    unsigned long long *accum;  // [M][N] fixed-point words, zero between launches
+    int N, K, M;
+    int kwords;          // K / 32
+    int nsets;           // look-up kernel: ceil(kwords / 8); matrix-core kernel: K-steps
+    int n_tiles;
+    int group_words;     // row-wise / uniform: words per alpha group
+    Divisor by_group_words;  // row / group_words
+    Divisor by_nsets;        // item / nsets
+    Divisor by_items;        // item / items_per_wg
+    int R;               // block modes: row groups
+    int rows_per_group;  // block modes: N / R
+    int nb;
+    int block_begin;     // grouped launches: first flat workgroup index of this problem
+    int mchunks;         // activation rows are handled in chunks
+    int n_blocks;        // workgroups of this problem in the flat grid
+    // Look-up kernel: the (tile, set) items of one row chunk, tile-major, are cut
+    // into `wgs_per_chunk` contiguous ranges of `items_per_wg` items.
+    int items_per_wg;
+    int wgs_per_chunk;
+    // Matrix-core kernel: K-steps per K-slice and slices per tile.
+    int sets_per_split;
+    int ksplit;
+    int finish;          // kFinishInline / kFinishDefer
+    // fused input transforms and output mode (row-wise look-up path only)
+    const __half *norm_w;  // non-null: the input is fp16(fp16(x * rsqrt(mean(x^2) + norm_eps)) * norm_w)
+    const __half *gate;    // non-null [M][K]: the input is fp16(fp16(silu(gate)) * x)
+    float norm_eps;
+    int overwrite;         // 1: out = y instead of out += y
+};
+
+struct Group {
+    int count;
+    Problem p[kMaxGroup];
+};
+
+__device__ __forceinline__ float half_bits_to_float(uint32_t bits16)
+{
+    return __half2float(__ushort_as_half((unsigned short)bits16));
+}
+
+__device__ __forceinline__ uint32_t float_to_half_bits(float f)
+{
+    return (uint32_t)__half_as_ushort(__float2half_rn(f));
+}
+
+// One partial sum as a contribution to an accumulator word: the addend, and the
+// flags to OR in first (0 for every finite partial sum within range).
+struct Contribution {
+    unsigned long long add, flags;
+};
+
+__device__ __forceinline__ Contribution fixed_contribution(float v)
+{
+    Contribution c;
+    c.flags = 0;
+    if (!(v <= 65536.0f)) c.flags |= kFlagPos;   // +inf, too large, NaN
+    if (!(v >= -65536.0f)) c.flags |= kFlagNeg;  // -inf, too small, NaN
+    v = c.flags ? 0.0f : v;
+    // rn(v * 2^31) without double arithmetic: v = hi + lo with hi = rn(v * 2^7) / 2^7 (an
+    // integer of at most 24 bits times 2^-7) and lo = v - hi (exact, |lo| <= 2^-8), so
+    // v * 2^31 = (hi * 2^7) * 2^24 + lo * 2^31, and only the second term needs rounding.
+    const float hi7 = rintf(v * 128.0f);
+    const float lo = fmaf(hi7, -1.0f / 128.0f, v);
+    const long long fx = ((long long)(int)hi7 << 24) + (long long)(int)rintf(lo * kFixedScaleF);
+    c.add = (unsigned long long)(fx + kBias) + kCountOne;
+    return c;
+}
+
+// The value of a complete accumulator word (`count` contributions).
+__device__ __forceinline__ float fixed_total(unsigned long long word, int count)
+{
+    const long long total = (long long)(word & kSumMask) - (long long)count * kBias;
+    float y = (float)((double)total * (1.0 / kFixedScale));
+    const bool pos = word & kFlagPos, neg = word & kFlagNeg;
+    if (pos || neg) y = (pos && neg) ? __builtin_nanf("") : pos ? __builtin_inff() : -__builtin_inff();
+    return y;
+}
+
+}  // namespace lutgemm
+
+#endif

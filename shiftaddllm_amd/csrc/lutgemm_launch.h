@@ -1,0 +1,22 @@
+// Launchers of the kernel templates, one translation unit per family so that the
+// library builds in parallel.  Each returns hipGetLastError() after the launch.
+#ifndef LUTGEMM_LAUNCH_H
+#define LUTGEMM_LAUNCH_H
+
+#include "lutgemm_common.h"
+
+namespace lutgemm {
+
+// look-up kernel, one problem; grid = (p.wgs_per_chunk, p.mchunks); mrows in {1, 2, 4}
+hipError_t launch_gemv_rowwise(const Problem &p, int mode, int mrows, hipStream_t stream);       // kRowF16, kUniformF16
+hipError_t launch_gemv_block(const Problem &p, int mode, int mrows, hipStream_t stream);         // kBlock*
+hipError_t launch_gemv_block_staged(const Problem &p, int mode, int mrows, hipStream_t stream);  // kBlock*Staged
+// look-up kernel, several row-wise problems, flat grid of `blocks` workgroups
+hipError_t launch_gemv_group(const Group &g, int xform, int blocks, hipStream_t stream);
+// matrix-core kernel; mt = 1 (16-row tiles) or 2 (32-row tiles)
+hipError_t launch_mfma(const Problem &p, int mt, hipStream_t stream);
+hipError_t launch_mfma_group(const Group &g, int mt, int blocks, hipStream_t stream);
+
+}  // namespace lutgemm
+
+#endif

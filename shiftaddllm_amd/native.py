@@ -29,6 +29,10 @@ C_ABI_SYMBOLS = (
     "lutgemm_gemv_block_apot_i8",
     "lutgemm_algorithmic_bytes",
     "lutgemm_copy_bytes",
+    "lutgemm_workspace_words",
+    "lutgemm_reserve_workspace",
+    "lutgemm_measure_stream_read",
+    "lutgemm_measure_empty_launch",
     "lutgemm_release_workspaces",
     "lutgemm_decode_rmsnorm_f16",
     "lutgemm_decode_attention_f16",
@@ -111,6 +115,14 @@ def cabi() -> ctypes.CDLL:
         lib.lutgemm_algorithmic_bytes.restype = sz
         lib.lutgemm_copy_bytes.argtypes = [vp, vp, sz, vp]
         lib.lutgemm_copy_bytes.restype = ci
+        lib.lutgemm_workspace_words.argtypes = [ci, ci]
+        lib.lutgemm_workspace_words.restype = sz
+        lib.lutgemm_reserve_workspace.argtypes = [vp, sz]
+        lib.lutgemm_reserve_workspace.restype = ci
+        lib.lutgemm_measure_stream_read.argtypes = [vp, sz, vp, vp]
+        lib.lutgemm_measure_stream_read.restype = ci
+        lib.lutgemm_measure_empty_launch.argtypes = [ci, vp]
+        lib.lutgemm_measure_empty_launch.restype = ci
         lib.lutgemm_release_workspaces.argtypes = []
         lib.lutgemm_release_workspaces.restype = ci
         lib.lutgemm_decode_rmsnorm_f16.argtypes = [vp, vp, vp, ci, ci, ctypes.c_float, vp, sz, vp]
