@@ -58,6 +58,8 @@ extern "C" {
 #define LUTGEMM_ENOMEM (-5)   /* workspace allocation failed                */
 #define LUTGEMM_ECAPTURE (-6) /* the stream is being captured and its workspace
                                  would have to grow: reserve it beforehand   */
+#define LUTGEMM_ETOOBIG (-7)  /* beyond the fixed buffer of the entry point
+                                 that does not allocate                      */
 
 /* Human-readable text for a return code (static storage). */
 const char *lutgemm_strerror(int code);
@@ -78,6 +80,26 @@ int lutgemm_last_hip_error(void);
 int lutgemm_gemv_rowwise_f16(const uint32_t *bW, const void *alpha_f16, const void *x_f16,
                              void *out_f16, int N, int K, int nb, int num_groups, int M,
                              void *stream);
+
+/*
+ * lutgemm_gemv_rowwise_f16 for callers that cannot allocate device memory: code
+ * under HIP graph capture, tight serving loops, harnesses that forbid it.  It
+ * has no counterpart in the reference.  Same arguments, semantics and results,
+ * but the accumulator words come from a fixed array inside the library
+ * (LUTGEMM_NOALLOC_MAX_WORDS words of 8 bytes = 2 MiB, which every GPU the
+ * library runs on holds until the process ends) instead of a per-stream
+ * workspace: the call never calls hipMalloc or hipFree and never synchronises.
+ * M * N may be at most LUTGEMM_NOALLOC_MAX_WORDS (LUTGEMM_ETOOBIG otherwise).
+ * All calls on one GPU share the array, whatever their stream, and each leaves
+ * the words it used at zero again: calls that overlap in time on one GPU race
+ * (order them, e.g. on one stream).  The first call on a device looks the
+ * array's address up, which may load the code object: make that call outside
+ * graph capture.
+ */
+#define LUTGEMM_NOALLOC_MAX_WORDS (1 << 18)
+int lutgemm_gemv_rowwise_f16_noalloc(const uint32_t *bW, const void *alpha_f16, const void *x_f16,
+                                     void *out_f16, int N, int K, int nb, int num_groups, int M,
+                                     void *stream);
 
 /*
  * Several row-wise-alpha GEMVs in ONE kernel launch.  No counterpart in the

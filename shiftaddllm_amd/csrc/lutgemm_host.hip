@@ -21,6 +21,7 @@ namespace {
 constexpr int kMfmaWaves = 8;       // waves of a matrix-core workgroup: K-steps of a round
 constexpr int kMfmaTileCols = 64;   // outputs per matrix-core workgroup
 constexpr int kMfmaStepK = 128;
+constexpr int kMaxDevices = 64;
 
 thread_local int g_last_hip_error = 0;
 
@@ -35,6 +36,32 @@ int hip_fail(hipError_t e)
 // (lutgemm_common.h).  Every launch leaves the words it used at zero, which is the
 // state the next launch needs, so launches that are ordered on a stream can share
 // one buffer.
+
+// Fixed buffer of the entry point that may not allocate.  Zero when the code object is
+// loaded; each GPU holds its own copy at its own address until the process ends.
+static __device__ __align__(256) unsigned long long scratch[LUTGEMM_NOALLOC_MAX_WORDS];
+
+std::mutex g_scratch_mutex;
+unsigned long long *g_scratch_ptr[kMaxDevices] = {};
+
+// Address of `scratch` on the current device, resolved once per device (in host code
+// the array's name is a stand-in, not a device address).
+int scratch_address(unsigned long long **out)
+{
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return hip_fail(e);
+    if (dev < 0 || dev >= kMaxDevices) return LUTGEMM_EUNSUP;
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {
+        void *ptr = nullptr;
+        e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+        if (e != hipSuccess) return hip_fail(e);
+        g_scratch_ptr[dev] = (unsigned long long *)ptr;
+    }
+    *out = g_scratch_ptr[dev];
+    return LUTGEMM_OK;
+}
 
 struct Workspace {
     unsigned long long *accum = nullptr;
@@ -86,11 +113,14 @@ int stream_workspace(hipStream_t stream, size_t words, unsigned long long **out)
 // Where a call takes its accumulator words from.
 struct Accum {
     hipStream_t stream;
+    bool fixed = false;  // the fixed device array instead of the stream's workspace
 };
 
 int accum_words(const Accum &a, size_t words, unsigned long long **out)
 {
-    return stream_workspace(a.stream, words, out);
+    if (!a.fixed) return stream_workspace(a.stream, words, out);
+    if (words > (size_t)LUTGEMM_NOALLOC_MAX_WORDS) return LUTGEMM_ETOOBIG;
+    return scratch_address(out);
 }
 
 int env_int(const char *name, int fallback)
@@ -447,6 +477,8 @@ const char *lutgemm_strerror(int code)
     case LUTGEMM_ECAPTURE:
         return "the stream is being captured and its workspace would have to grow "
                "(call lutgemm_reserve_workspace before capturing)";
+    case LUTGEMM_ETOOBIG:
+        return "M * N exceeds LUTGEMM_NOALLOC_MAX_WORDS, the fixed buffer of the entry point that does not allocate";
     default: return "unknown lutgemm error";
     }
 }
@@ -459,6 +491,19 @@ int lutgemm_gemv_rowwise_f16(const uint32_t *bW, const void *alpha_f16, const vo
 {
     return run(kRowF16, bW, alpha_f16, nullptr, x_f16, out_f16, N, K, nb, num_groups, M,
                Accum{(hipStream_t)stream});
+}
+
+int lutgemm_gemv_rowwise_f16_noalloc(const uint32_t *bW, const void *alpha_f16, const void *x_f16,
+                                     void *out_f16, int N, int K, int nb, int num_groups, int M,
+                                     void *stream)
+{
+    if (N > 0 && M > 0 && (size_t)N * (size_t)M > (size_t)LUTGEMM_NOALLOC_MAX_WORDS) return LUTGEMM_ETOOBIG;
+    // set-up on the first call on a device, whether or not this call needs the words
+    unsigned long long *unused = nullptr;
+    const int rc = scratch_address(&unused);
+    if (rc != LUTGEMM_OK) return rc;
+    return run(kRowF16, bW, alpha_f16, nullptr, x_f16, out_f16, N, K, nb, num_groups, M,
+               Accum{(hipStream_t)stream, true});
 }
 
 int lutgemm_gemv_rowwise_f16_grouped(int count, const lutgemm_rowwise_problem *problems,

@@ -21,6 +21,7 @@ C_ABI_SYMBOLS = (
     "lutgemm_strerror",
     "lutgemm_last_hip_error",
     "lutgemm_gemv_rowwise_f16",
+    "lutgemm_gemv_rowwise_f16_noalloc",
     "lutgemm_gemv_rowwise_f16_grouped",
     "lutgemm_gemv_rowwise_f16_fused",
     "lutgemm_gemv_uniform_f16",
@@ -41,6 +42,7 @@ C_ABI_SYMBOLS = (
 
 
 MAX_GROUP = 8
+NOALLOC_MAX_WORDS = 1 << 18
 
 
 class RowwiseProblem(ctypes.Structure):
@@ -100,6 +102,8 @@ def cabi() -> ctypes.CDLL:
         lib.lutgemm_last_hip_error.argtypes = []
         lib.lutgemm_last_hip_error.restype = ci
         lib.lutgemm_gemv_rowwise_f16.argtypes = [vp, vp, vp, vp, ci, ci, ci, ci, ci, vp]
+        lib.lutgemm_gemv_rowwise_f16_noalloc.argtypes = [vp, vp, vp, vp, ci, ci, ci, ci, ci, vp]
+        lib.lutgemm_gemv_rowwise_f16_noalloc.restype = ci
         lib.lutgemm_gemv_rowwise_f16_grouped.argtypes = [ci, ctypes.POINTER(RowwiseProblem), vp]
         lib.lutgemm_gemv_rowwise_f16_grouped.restype = ci
         lib.lutgemm_gemv_rowwise_f16_fused.argtypes = [ci, ctypes.POINTER(FusedProblem), vp]
