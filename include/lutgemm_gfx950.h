@@ -21,9 +21,9 @@
  *           (mv_fp16_bias.hpp:101,216,324,491,577; lut_gemm/quant.py:46).
  *           Unlike the reference's fp16 atomics the sum is formed in fp32 and
  *           rounded to fp16 once, and it is deterministic.
- *           A sum that is not finite comes out as it would from IEEE
- *           arithmetic (NaN stays NaN, +inf and -inf give NaN), whatever the
- *           launch plan; partial sums beyond +-65536 count as infinite.
+ *           A NaN input gives NaN and an infinite input gives an infinity
+ *           or NaN in every output it reaches, whatever the launch plan
+ *           (partial sums beyond +-65536 count as infinite).
  * Shape rules enforced here (the reference checks nothing and reads or writes
  * out of bounds instead): K % 32 == 0, N % 4 == 0, 1 <= nb <= 4,
  * 1 <= M <= 65535, 16-byte aligned bW and x, 8-byte aligned row-wise alpha and out.
@@ -271,7 +271,8 @@ int lutgemm_decode_rmsnorm_f16(const void *x, const void *weight, void *y, int r
  * [batch][kv_heads*head_dim], out [batch][heads*head_dim]; heads a multiple of
  * kv_heads; head_dim a multiple of 8, at most 256; max_positions at most 8192.
  * `position` is a DEVICE pointer so that a captured graph can be replayed for
- * successive tokens. */
+ * successive tokens; the kernel clamps *position into 0..max_positions-1 (it
+ * cannot report an error), so the caller must keep it inside the cache. */
 int lutgemm_decode_attention_f16(const void *q, const void *k, const void *v, const void *cos_table,
                                  const void *sin_table, void *k_cache, void *v_cache, const int64_t *position,
                                  void *out, int batch, int heads, int kv_heads, int head_dim, int max_positions,

@@ -316,6 +316,10 @@ class LutDecoder(nn.Module):
 
     @torch.no_grad()
     def forward_token(self, ids: torch.Tensor, position: int):
+        # the attention kernel clamps the position into the cache: past its end it would
+        # overwrite the last slot and return plausible but wrong logits
+        if not 0 <= position < self.cfg.max_positions:
+            raise ValueError(f"position {position} outside the KV cache of {self.cfg.max_positions} positions")
         self.ids.copy_(ids)
         self.pos.fill_(position)
         if self._graph is not None:

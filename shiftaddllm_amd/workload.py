@@ -55,7 +55,11 @@ def assign_signs(w: torch.Tensor, alpha: torch.Tensor, chunk_rows: int = 1 << 15
     for r0 in range(0, rows, chunk_rows):
         r1 = min(rows, r0 + chunk_rows)
         values = alpha[r0:r1].float().mm(book.t())           # [r, C]
-        vs, order = torch.sort(values)
+        # Equal code values are common (two planes with the same power-of-two scale): the
+        # CPU sort the reference runs on keeps their order; asked for explicitly so that a
+        # GPU breaks those ties the same way (otherwise it picks other, equivalent signs
+        # and the next refinement round drifts off the reference's bits).
+        vs, order = torch.sort(values, stable=True)
         mids = (vs[:, :-1] + vs[:, 1:]) / 2                  # non-decreasing
         slot = torch.searchsorted(mids, w[r0:r1].float().contiguous(), right=True)   # mids <= w
         out[r0:r1] = book8[torch.gather(order, 1, slot)]
