@@ -5,14 +5,21 @@ Workload (the configuration the headline metric is quoted on): the seven linear 
 decoder block as 3-bit BCQ LUT-GEMVs (group 128 along K, power-of-two alphas,
 batch 1).  One *step* is one decoded token's worth of them: 32 blocks x 7
 GEMVs = 224 launches streaming 2.74 GB of distinct weights (so nothing is
-served from the 256 MB Infinity Cache), replayed from one HIP graph.
+served from the 256 MB Infinity Cache), replayed from one HIP graph, one launch
+per GEMV through the drop-in entry point, one after the other on one stream.
 
-Prints ONE JSON line.  `value` is the mean device time per GEMV call in that
-sequence, in microseconds, with all operands resident in HBM.  `roofline`
-prices the same launches against the 8 TB/s HBM peak using the algorithmic
-bytes per call (signs + alphas + x + y read + y write).  `cpu_baseline` is the
-reference's CPU-executable path (dequantise once, fp32 linear) timed on this
-box's host cores on one decoder block.
+Prints ONE JSON line.  `value` is the step's device time divided by its 224
+calls, in microseconds, with all operands resident in HBM.  `roofline` prices
+the same launches: algorithmic bytes per launch (signs + alphas + x + y read +
+y write) over the mean launch duration, against the 8 TB/s HBM peak, with the
+measured floors beside it (an empty launch, and a kernel that only streams the
+sign words).  `dependency_branches` is the same step with q|k|v and gate|up of a
+block on parallel graph branches (slower here: the fork and join nodes cost more
+than the overlap gains).  `configs` holds every other BASELINE configuration (us per call over
+rotating weights, GB/s, fraction of peak, error against the CPU oracle where the
+oracle is affordable, a CPU time for one shape per configuration).
+`cpu_baseline` is the reference's CPU-executable path (dequantise once, fp32
+linear) timed on this box's host cores on one decoder block.
 
 Run with no arguments for the default configuration; `--gpus` above 1 is
 refused (this build is single-GPU).
@@ -35,6 +42,7 @@ HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
 N_LAYERS = 32
 NB, GROUP = 3, 128
 TRAFFIC_NOTE = os.path.join(REPO, "profiles", "lut_gemv_llama7b_3bit_pmc.md")
+DATA_NOTE = "random sign words, power-of-two alphas halving per bit plane, x ~ N(0,1) fp16 (timing does not depend on the data: look-ups are conflict-free by construction)"
 
 
 def parse_args():
@@ -46,13 +54,13 @@ def parse_args():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying a HIP graph")
     ap.add_argument("--no-decode", action="store_true", help="skip the full-model decode runs (config 4)")
-    ap.add_argument("--no-shape-table", action="store_true", help="skip timing every shape alone")
+    ap.add_argument("--no-configs", action="store_true", help="skip the table of the other configurations")
     ap.add_argument("--plain-only", action="store_true",
-                    help="only the 224-launch step (no fused sequences, no per-shape table): for profiler runs")
+                    help="only the 224 launches one after the other (no branches, no fused sequences, no tables): for profiler runs")
     ap.add_argument("--profile-shape", type=str, default="",
                     help="N,K[,nb[,iters[,M]]]: only launch this shape repeatedly (for rocprofv3 runs) and exit")
-    ap.add_argument("--batch-table", action="store_true",
-                    help="only time the 70B and 7B shapes over 1..32 activation rows (graph replay, rotating weights) and exit")
+    ap.add_argument("--profile-floor", type=str, default="",
+                    help="N,K[,nb[,iters]]: only launch the floor kernels for this shape (empty launch; stream-read of the sign words) and exit")
     ap.add_argument("--profile-decode", type=int, default=0,
                     help="batch: only replay ten graph-captured decode steps of the 7B decoder (for rocprofv3 runs) and exit")
     ap.add_argument("--profile-copy", type=int, default=0,
@@ -98,17 +106,67 @@ def main():
     dev = torch.device("cuda:0")
     lib = native.cabi()            # raises if the HIP library is not built: no fallback
     launch = lib.lutgemm_gemv_rowwise_f16
+    vp = lambda t: ctypes.c_void_p(t.data_ptr())
 
-    def run(g, stream_ptr):
-        rc = launch(*g.args(), stream_ptr)
+    def check(rc):
         if rc:
             raise RuntimeError(lib.lutgemm_strerror(rc).decode())
 
+    def run(g, stream_ptr):
+        check(launch(*g.args(), stream_ptr))
+
     def alg_bytes(g):
-        return lib.lutgemm_algorithmic_bytes(g.N, g.K, g.nb, 1, g.groups * g.nb * g.N, 2)
+        return lib.lutgemm_algorithmic_bytes(g.N, g.K, g.nb, g.M, g.groups * g.nb * g.N, 2)
 
     stream = torch.cuda.Stream()
     sp = ctypes.c_void_p(stream.cuda_stream)
+
+    def capture(fn, warm=True):
+        """fn() issues launches on `stream`; returns a graph of them (None with --no-graph)."""
+        torch.cuda.synchronize()                  # operands may have been made on another stream
+        if warm:
+            with torch.cuda.stream(stream):
+                fn()                              # sizes this stream's workspace before any capture
+            stream.synchronize()
+        if args.no_graph:
+            return None
+        gr = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(gr, stream=stream):
+            fn()
+        return gr
+
+    def timed(fn, gr, steps, warmup):
+        """(wall ms/step, device ms/step): wall clock between synchronisations and
+        HIP events recorded on the launch stream around the same region."""
+        def step():
+            with torch.cuda.stream(stream):
+                if gr is not None:
+                    gr.replay()
+                else:
+                    fn()
+        for _ in range(warmup):
+            step()
+        torch.cuda.synchronize()
+        ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        t_start = time.perf_counter()
+        with torch.cuda.stream(stream):
+            ev0.record(stream)
+        for _ in range(steps):
+            step()
+        with torch.cuda.stream(stream):
+            ev1.record(stream)
+        torch.cuda.synchronize()
+        wall = (time.perf_counter() - t_start) * 1e3 / steps
+        return wall, ev0.elapsed_time(ev1) / steps
+
+    def us_per_call(seq_fn, n_calls, reps=3):
+        """Median device time per call of a sequence replayed from a graph."""
+        gr = capture(seq_fn)
+        ts = []
+        for _ in range(reps):
+            _, dms = timed(seq_fn, gr, 1, 1)
+            ts.append(dms * 1e3 / n_calls)
+        return statistics.median(ts)
 
     # ---- profiler helper modes --------------------------------------------
     if args.profile_copy:
@@ -117,98 +175,25 @@ def main():
         dst = torch.empty_like(src)
         with torch.cuda.stream(stream):
             for _ in range(5):
-                lib.lutgemm_copy_bytes(ctypes.c_void_p(dst.data_ptr()), ctypes.c_void_p(src.data_ptr()), nbytes, sp)
+                lib.lutgemm_copy_bytes(vp(dst), vp(src), nbytes, sp)
         stream.synchronize()
         print(json.dumps({"copy_bytes": nbytes, "launches": 5}))
         return
-    if args.batch_table:
-        table = {}
-        shapes = [(8192, 8192, 2), (8192, 8192, 4), (28672, 8192, 2), (28672, 8192, 4), (8192, 28672, 4),
-                  (1024, 8192, 4), (4096, 4096, 3), (3072, 768, 3)]     # last: OPT-125m fc1 (config 1)
-        for (N, K, nb) in shapes:
-            row = {}
-            for M in (1, 2, 4, 8, 16, 32):
-                cnt = max(3, min(24, (400 << 20) // (K // 8 * N * nb)))     # distinct weight sets: > 256 MB in rotation
-                pool = [Gemv(torch, dev, N, K, nb, 7 * i + M, M=M) for i in range(cnt)]
-                with torch.cuda.stream(stream):
-                    run(pool[0], sp)                                         # sizes the stream's workspace
-                stream.synchronize()
-                seq = (pool * ((24 + cnt - 1) // cnt))[:max(24, cnt)]
-                gr = torch.cuda.CUDAGraph()
-                with torch.cuda.graph(gr, stream=stream):
-                    for g in seq:
-                        run(g, sp)
-                ts = []
-                for _ in range(3):
-                    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-                    with torch.cuda.stream(stream):
-                        e0.record(stream)
-                        gr.replay()
-                        e1.record(stream)
-                    torch.cuda.synchronize()
-                    ts.append(e0.elapsed_time(e1) * 1e3 / len(seq))
-                us = statistics.median(ts)
-                byts = lib.lutgemm_algorithmic_bytes(N, K, nb, M, (K // GROUP) * nb * N, 2)
-                row[f"M{M}"] = {"us_per_call": round(us, 1), "GBps": round(byts / us / 1e3),
-                                "dense_equiv_TFLOPs": round(2 * M * N * K / us / 1e6, 1)}
-                del pool, seq, gr
-            table[f"{N}x{K}x{nb}bit"] = row
-        # config 3: Llama-2-13B shapes, 2-bit, block alpha (8 row groups), one row, every storage format
-        block = {}
-        entry = {"f16": lib.lutgemm_gemv_block_f16, "apot_i8": lib.lutgemm_gemv_block_apot_i8,
-                 "shift_u16": lib.lutgemm_gemv_block_shift_u16}
-        vp = lambda t: ctypes.c_void_p(t.data_ptr())
-        for (N, K) in workload.LLAMA2_13B_SHAPES:
-            nb, R = 2, 8
-            row = {}
-            for kind, fn in entry.items():
-                cnt = max(4, min(40, (500 << 20) // (K // 8 * N * nb)))
-                pool = []
-                for i in range(cnt):
-                    g = torch.Generator(device=dev).manual_seed(17 * i + N)
-                    bW = torch.randint(-2 ** 31, 2 ** 31 - 1, (K // 32, nb, N), generator=g, device=dev, dtype=torch.int32)
-                    e = (torch.randint(-9, -5, (K // 8, 1, R), generator=g, device=dev).float()
-                         - torch.arange(nb, device=dev).float().view(1, nb, 1))
-                    if kind == "f16":
-                        alpha = torch.exp2(e).half().contiguous()
-                    elif kind == "apot_i8":
-                        alpha = torch.full((K // 8, nb, R, 3), -128, dtype=torch.int8, device=dev)
-                        alpha[..., 0] = e.to(torch.int8)
-                    else:
-                        alpha = torch.randint(0, 512, (K // 8, nb, R), generator=g, device=dev).to(torch.int16)
-                    pool.append((bW, alpha, torch.randn((1, K), generator=g, device=dev).half(),
-                                 torch.zeros((1, N), dtype=torch.float16, device=dev)))
-
-                def go(o, fn=fn, kind=kind, N=N, K=K):
-                    extra = () if kind == "f16" else (3,)
-                    rc = fn(vp(o[0]), vp(o[1]), vp(o[2]), vp(o[3]), N, K, nb, R, *extra, 1, sp)
-                    if rc:
-                        raise RuntimeError(lib.lutgemm_strerror(rc).decode())
-                with torch.cuda.stream(stream):
-                    go(pool[0])
-                stream.synchronize()
-                seq = (pool * 3)[:max(40, cnt)]
-                gr = torch.cuda.CUDAGraph()
-                with torch.cuda.graph(gr, stream=stream):
-                    for o in seq:
-                        go(o)
-                ts = []
-                for _ in range(3):
-                    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-                    with torch.cuda.stream(stream):
-                        e0.record(stream)
-                        gr.replay()
-                        e1.record(stream)
-                    torch.cuda.synchronize()
-                    ts.append(e0.elapsed_time(e1) * 1e3 / len(seq))
-                us = statistics.median(ts)
-                byts = lib.lutgemm_algorithmic_bytes(N, K, nb, 1, pool[0][1].numel(), pool[0][1].element_size())
-                row[kind] = {"us_per_call": round(us, 2), "GBps": round(byts / us / 1e3)}
-                del pool, seq, gr
-            block[f"{N}x{K}x{nb}bit_R{R}"] = row
-        print(json.dumps({"batch_table": table, "block_alpha_13b": block, "note": "one launch per call, HIP-graph replay of 24 calls over "
-                          "rotating weights, median of 3; 1 row (and 2 rows above 32 MB of signs) = table look-up "
-                          "kernel, otherwise matrix-core kernel"}))
+    if args.profile_floor:
+        parts = [int(v) for v in args.profile_floor.split(",")]
+        N, K = parts[0], parts[1]
+        nb = parts[2] if len(parts) > 2 else NB
+        iters = parts[3] if len(parts) > 3 else 8
+        nbytes = K // 8 * N * nb
+        pool = [torch.empty(nbytes, dtype=torch.uint8, device=dev).random_(0, 255) for _ in range(iters)]
+        torch.cuda.synchronize()
+        with torch.cuda.stream(stream):
+            for _ in range(iters):
+                check(lib.lutgemm_measure_empty_launch(512, sp))
+            for buf in pool:          # each launch streams bytes never read before
+                check(lib.lutgemm_measure_stream_read(vp(buf), nbytes, None, sp))
+        stream.synchronize()
+        print(json.dumps({"shape": [N, K, nb], "launches_each": iters, "sign_bytes_per_launch": nbytes}))
         return
     if args.profile_decode:
         from shiftaddllm_amd import decode
@@ -257,14 +242,14 @@ def main():
     import oracle
     parity = {}
     torch.cuda.synchronize()                  # pool tensors were made on the default stream
-    for g in pool[3:7]:                       # o_proj, gate, up, down of block 0
+    for g in pool[0:1] + pool[3:7]:           # q_proj, o_proj, gate, up, down of block 0: every shape of the block
         with torch.cuda.stream(stream):
             g.out.zero_()
             run(g, sp)
         stream.synchronize()
         want, _ = oracle.gemv_rowwise_c(g.bW.cpu().numpy(), g.alpha.cpu().numpy(), g.x.cpu().numpy(), g.groups)
         rel, mad = oracle.error_metrics(g.out.float().cpu().numpy(), want.astype(np.float32))
-        parity[f"{g.N}x{g.K}"] = {"rel_l2": rel, "max_rel": mad}
+        parity.setdefault(f"{g.N}x{g.K}", {"rel_l2": rel, "max_rel": mad})
         if rel > 2e-3 or mad > 1e-2:
             raise SystemExit(f"parity failure on {g.N}x{g.K}: rel_l2={rel} max={mad}")
 
@@ -279,9 +264,7 @@ def main():
         return arr
 
     def run_group(arr):
-        rc = grouped(len(arr), arr, sp)
-        if rc:
-            raise RuntimeError(lib.lutgemm_strerror(rc).decode())
+        check(grouped(len(arr), arr, sp))
 
     blocks = [pool[i:i + 7] for i in range(0, len(pool), 7)]
     # dependency-respecting fusion inside a decoder block: [q,k,v] [o] [gate,up] [down]
@@ -293,6 +276,35 @@ def main():
         for g in pool:
             run(g, sp)
 
+    # One launch per GEMV with the dependencies of a decoder block: q, k, v fork onto two
+    # side streams and join before o; gate and up likewise before down.  Every stream has
+    # the default priority and its own accumulator workspace (reserved up front, since a
+    # stream under capture cannot grow it).
+    side = [torch.cuda.Stream(), torch.cuda.Stream()]
+    side_ptr = [ctypes.c_void_p(s.cuda_stream) for s in side]
+    for s in side_ptr:
+        check(lib.lutgemm_reserve_workspace(s, lib.lutgemm_workspace_words(11008, 1)))
+
+    def fork(gemvs):
+        """gemvs[0] on the main stream, the others on side streams, joined afterwards."""
+        ev = torch.cuda.Event()
+        ev.record(stream)
+        for s, sptr, g in zip(side, side_ptr, gemvs[1:]):
+            s.wait_event(ev)
+            run(g, sptr)
+        run(gemvs[0], sp)
+        for s, _ in zip(side, gemvs[1:]):
+            done = torch.cuda.Event()
+            done.record(s)
+            stream.wait_event(done)
+
+    def seq_branched():
+        for b in blocks:
+            fork(b[0:3])
+            run(b[3], sp)
+            fork(b[4:6])
+            run(b[6], sp)
+
     def seq_fused(groups):
         def f():
             for blk in groups:
@@ -300,58 +312,66 @@ def main():
                     run_group(arr)
         return f
 
-    def capture(fn):
-        with torch.cuda.stream(stream):
-            fn()                              # sizes this stream's workspace before any capture
-        stream.synchronize()
-        if args.no_graph:
-            return None
-        gr = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(gr, stream=stream):
-            fn()
-        return gr
-
-    def timed(fn, gr, steps, warmup):
-        """(wall ms/step, device ms/step): wall clock between synchronisations and
-        HIP events recorded on the launch stream around the same region."""
-        def step():
-            with torch.cuda.stream(stream):
-                if gr is not None:
-                    gr.replay()
-                else:
-                    fn()
-        for _ in range(warmup):
-            step()
-        torch.cuda.synchronize()
-        ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        t_start = time.perf_counter()
-        with torch.cuda.stream(stream):
-            ev0.record(stream)
-        for _ in range(steps):
-            step()
-        with torch.cuda.stream(stream):
-            ev1.record(stream)
-        torch.cuda.synchronize()
-        wall = (time.perf_counter() - t_start) * 1e3 / steps
-        return wall, ev0.elapsed_time(ev1) / steps
-
-    # ---- the timed step: 224 separate launches, the drop-in call pattern -----------
     props = torch.cuda.get_device_properties(dev)
     device_info = {"name": props.name, "compute_units": props.multi_processor_count,
                    "hbm_GiB": round(props.total_memory / 2 ** 30)}
-    graph = capture(seq_plain)
+    graph_plain = capture(seq_plain)
     # Power management follows sustained load: run the step untimed for about a second
     # first, whatever --warmup says; the W warm-up steps follow.  (Runs on different
-    # boxes of the same pool still differ by about 5 % on the K-split-heavy shapes.)
+    # boxes of the same pool still differ by about 10 % on the K-split-heavy shapes.)
     t_ramp = time.perf_counter()
     while time.perf_counter() - t_ramp < 1.0:
         with torch.cuda.stream(stream):
             for _ in range(20):
-                graph.replay() if graph is not None else seq_plain()
+                graph_plain.replay() if graph_plain is not None else seq_plain()
         torch.cuda.synchronize()
-    ms_per_step, dev_ms_per_step = timed(seq_plain, graph, args.steps, args.warmup)
-    us_per_call = dev_ms_per_step * 1e3 / calls_per_step
+    # ---- the timed step: 224 launches strictly one after the other --------------------
+    ms_per_step, dev_ms_per_step = timed(seq_plain, graph_plain, args.steps, args.warmup)
+    step_kind = "one after the other on one stream"
+    # ---- the same launches with the dependencies of a decoder block as graph branches ----
+    branched = None
+    if not args.plain_only:
+        graph_br = capture(seq_branched)
+        _, br_ms = timed(seq_branched, graph_br, args.steps, args.warmup)
+        branched = {"what": "q|k|v and gate|up of a block on parallel graph branches (two side streams, default "
+                            "priority), o and down after their joins, blocks one after the other",
+                    "device_ms_per_step": round(br_ms, 5), "us_per_call": round(br_ms * 1e3 / calls_per_step, 4)}
+        # parity of the branched step against separate launches (bit-identical: same kernels and plans)
+        with torch.cuda.stream(stream):
+            for g in pool[:7]:
+                g.out.zero_()
+            for g in pool[:7]:
+                run(g, sp)
+        stream.synchronize()
+        ref7 = [g.out.clone() for g in pool[:7]]
+        for g in pool:
+            g.out.zero_()
+        torch.cuda.synchronize()
+        with torch.cuda.stream(stream):
+            graph_br.replay() if graph_br is not None else seq_branched()
+        torch.cuda.synchronize()
+        parity["branched_equals_serial"] = all(torch.equal(a, g.out) for a, g in zip(ref7, pool[:7]))
+        if not parity["branched_equals_serial"]:
+            raise SystemExit("branched step disagrees with separate launches")
+    value_us = dev_ms_per_step * 1e3 / calls_per_step
     achieved_gbs = step_bytes / (dev_ms_per_step * 1e-3) / 1e9
+
+    # ---- floors: an empty launch and a kernel that only streams the sign words --------
+    floors = None
+    if not args.plain_only:
+        floors = {}
+        floors["empty_launch_us"] = round(us_per_call(
+            lambda: [check(lib.lutgemm_measure_empty_launch(512, sp)) for _ in range(64)], 64), 3)
+        rd = torch.empty(3 << 30, dtype=torch.uint8, device=dev).random_(0, 255)
+        torch.cuda.synchronize()
+        for (N, K, nb) in ((4096, 4096, 3), (11008, 4096, 3), (8192, 8192, 4), (28672, 8192, 4)):
+            nbytes = K // 8 * N * nb
+            cnt = min(64, (3 << 30) // nbytes)
+            ptrs = [ctypes.c_void_p(rd.data_ptr() + i * nbytes) for i in range(cnt)]
+            us = us_per_call(lambda: [check(lib.lutgemm_measure_stream_read(pt, nbytes, None, sp)) for pt in ptrs], cnt)
+            floors[f"stream_read_{N}x{K}x{nb}bit_us"] = round(us, 3)
+        del rd
+        torch.cuda.empty_cache()
 
     # ---- the same step with fused launches --------------------------------------------
     fused = {}
@@ -387,55 +407,175 @@ def main():
         if worst > 2e-4:
             raise SystemExit(f"fused launch disagrees with separate launches: rel_l2={worst}")
 
-    # ---- every shape alone: hot (one buffer, cache resident) and rotating (HBM) --------
+    # ---- every 7B shape alone: hot (one buffer, cache resident) and rotating (HBM) -----
     shape_table = None
-    if not (args.no_shape_table or args.plain_only):
+    if not args.plain_only:
         shape_table = {}
         for (N, K) in ((4096, 4096), (11008, 4096), (4096, 11008)):
             same = [g for g in pool if (g.N, g.K) == (N, K)]
             row = {}
             for label, seq in (("hot", [same[0]] * 64), ("rotating", (same * 8)[:max(64, len(same))])):
-                def f(seq=seq):
-                    for g in seq:
-                        run(g, sp)
-                gr = capture(f)
-                _, dms = timed(f, gr, 7, 2)
-                us = dms * 1e3 / len(seq)
+                us = us_per_call(lambda seq=seq: [run(g, sp) for g in seq], len(seq))
                 row[label] = {"us_per_call": round(us, 3), "GBps": round(same[0].bytes / us / 1e3, 1),
                               "frac_hbm_peak": round(same[0].bytes / us / 1e3 / HBM_PEAK_GBS, 4)}
             row["algorithmic_bytes"] = same[0].bytes
+            if floors:
+                row["stream_read_floor_us"] = floors.get(f"stream_read_{N}x{K}x3bit_us", floors.get("stream_read_11008x4096x3bit_us"))
             shape_table[f"{N}x{K}"] = row
 
     # ---- CPU baseline: dequantise once + fp32 linear on host cores ----------
-    cpu = None
-    if not args.no_cpu_baseline:
-        threads = torch.get_num_threads()
-        block = pool[:7]
-        runs = []
-        for g in block:
-            f, _ = oracle.cpu_dense_path(g.bW.cpu().numpy(), g.alpha.cpu().numpy())
-            runs.append((f, g.x.cpu()))
+    def cpu_time(runs, budget_s, max_samples=10):
         for f, x in runs:
             f(x)
         samples = []
-        t_lim = time.time() + 20.0
-        while len(samples) < 10 and time.time() < t_lim:
+        t_lim = time.time() + budget_s
+        while len(samples) < 3 or (len(samples) < max_samples and time.time() < t_lim):
             t = time.perf_counter()
             for f, x in runs:
                 f(x)
             samples.append((time.perf_counter() - t) / len(runs))
-        cpu = {"value": round(statistics.median(samples) * 1e6, 1), "unit": "us/call", "cores": threads,
-               "kind": "port",
-               "sample": f"one decoder block (7 GEMVs of this workload), weights dequantised once, fp32 "
-                         f"torch linear, median of {len(samples)} passes; host shows {os.cpu_count()} cpus"}
+        return statistics.median(samples) * 1e6, len(samples)
 
-    launch_mode = "eager" if graph is None else "hip-graph replay"
+    cpu = None
+    threads = torch.get_num_threads()
+    if not args.no_cpu_baseline:
+        runs = []
+        for g in pool[:7]:
+            f, _ = oracle.cpu_dense_path(g.bW.cpu().numpy(), g.alpha.cpu().numpy())
+            runs.append((f, g.x.cpu()))
+        us, n = cpu_time(runs, 12.0)
+        cpu = {"value": round(us, 1), "unit": "us/call", "cores": threads, "kind": "port",
+               "sample": f"one decoder block (7 GEMVs of this workload), weights dequantised once, fp32 "
+                         f"torch linear, median of {n} passes; host shows {os.cpu_count()} cpus"}
+        del runs
+
+    launch_mode = "eager" if args.no_graph else "hip-graph replay"
+    del blocks, fused4, fused1, graph_plain
+    keep = pool[:7]
+    del pool
+    torch.cuda.empty_cache()
+
+    # ---- the other configurations: one launch per call, rotating weights -----------------
+    configs = None
+    if not (args.no_configs or args.plain_only):
+        configs = {"note": "us per call = device time of a HIP-graph replay of >= 24 calls over distinct weight sets "
+                           "(> 256 MB in rotation), median of 3; 1 row (and 2 rows above 32 MB of signs) = table look-up "
+                           "kernel, otherwise matrix-core kernel; " + DATA_NOTE}
+
+        def row_entry(N, K, nb, M, with_oracle):
+            cnt = max(3, min(24, (400 << 20) // (K // 8 * N * nb)))
+            gp = [Gemv(torch, dev, N, K, nb, 7 * i + M + N, M=M) for i in range(cnt)]
+            seq = (gp * ((24 + cnt - 1) // cnt))[:max(24, cnt)]
+            us = us_per_call(lambda: [run(g, sp) for g in seq], len(seq))
+            byts = alg_bytes(gp[0])
+            e = {"us_per_call": round(us, 2), "tokens_per_s": round(M * 1e6 / us), "GBps": round(byts / us / 1e3),
+                 "frac_hbm_peak": round(byts / us / 1e3 / HBM_PEAK_GBS, 4)}
+            if M > 1:
+                e["dense_equiv_TFLOPs"] = round(2 * M * N * K / us / 1e6, 1)
+            if with_oracle:
+                g = gp[0]
+                with torch.cuda.stream(stream):
+                    g.out.zero_()
+                    run(g, sp)
+                stream.synchronize()
+                want, _ = oracle.gemv_rowwise_c(g.bW.cpu().numpy(), g.alpha.cpu().numpy(), g.x.cpu().numpy(), g.groups)
+                e["rel_l2_vs_oracle"] = float(f"{oracle.error_metrics(g.out.float().cpu().numpy(), want.astype(np.float32))[0]:.3e}")
+                if e["rel_l2_vs_oracle"] > 2e-3:
+                    raise SystemExit(f"parity failure on {N}x{K}x{nb} M={M}")
+            first = gp[0]
+            del gp, seq
+            return e, first
+
+        # config 1: OPT-125m fc1
+        N, K = workload.OPT125M_FC1
+        e, g1 = row_entry(N, K, 3, 1, True)
+        if not args.no_cpu_baseline:
+            f, _ = oracle.cpu_dense_path(g1.bW.cpu().numpy(), g1.alpha.cpu().numpy())
+            us, n = cpu_time([(f, g1.x.cpu())], 2.0)
+            e["cpu_us_per_call"] = round(us, 1)
+        configs["config1_opt125m_fc1_3072x768x3bit"] = e
+
+        # config 3: Llama-2-13B shapes, 2-bit, block alpha (8 row groups), one row, every storage format
+        entry = {"f16": lib.lutgemm_gemv_block_f16, "apot_i8": lib.lutgemm_gemv_block_apot_i8,
+                 "shift_u16": lib.lutgemm_gemv_block_shift_u16}
+        okind = {"f16": oracle.ALPHA_F16, "apot_i8": oracle.ALPHA_APOT_I8, "shift_u16": oracle.ALPHA_SHIFT_U16}
+        c3 = {}
+        for (N, K) in workload.LLAMA2_13B_SHAPES:
+            nb, R = 2, 8
+            row = {}
+            for kind, fn in entry.items():
+                cnt = max(4, min(40, (500 << 20) // (K // 8 * N * nb)))
+                bp = []
+                for i in range(cnt):
+                    g = torch.Generator(device=dev).manual_seed(17 * i + N)
+                    bW = torch.randint(-2 ** 31, 2 ** 31 - 1, (K // 32, nb, N), generator=g, device=dev, dtype=torch.int32)
+                    ee = (torch.randint(-9, -5, (K // 8, 1, R), generator=g, device=dev).float()
+                          - torch.arange(nb, device=dev).float().view(1, nb, 1))
+                    xs = 1.0
+                    if kind == "f16":
+                        alpha = torch.exp2(ee).half().contiguous()
+                    elif kind == "apot_i8":
+                        alpha = torch.full((K // 8, nb, R, 3), -128, dtype=torch.int8, device=dev)
+                        alpha[..., 0] = ee.to(torch.int8)
+                    else:
+                        alpha = torch.randint(0, 512, (K // 8, nb, R), generator=g, device=dev).to(torch.int16)
+                        xs = 0.002          # multipliers reach 384: keep outputs inside fp16
+                    bp.append((bW, alpha, (torch.randn((1, K), generator=g, device=dev) * xs).half(),
+                               torch.zeros((1, N), dtype=torch.float16, device=dev)))
+
+                def go(o, fn=fn, kind=kind, N=N, K=K):
+                    extra = () if kind == "f16" else (3,)
+                    check(fn(vp(o[0]), vp(o[1]), vp(o[2]), vp(o[3]), N, K, nb, R, *extra, 1, sp))
+                seq = (bp * 3)[:max(40, cnt)]
+                us = us_per_call(lambda: [go(o) for o in seq], len(seq))
+                byts = lib.lutgemm_algorithmic_bytes(N, K, nb, 1, bp[0][1].numel() // (3 if kind == "apot_i8" else 1),
+                                                     3 if kind == "apot_i8" else 2)
+                o = bp[0]
+                with torch.cuda.stream(stream):
+                    o[3].zero_()
+                    go(o)
+                stream.synchronize()
+                want, _ = oracle.gemv_block_c(o[0].cpu().numpy(), o[1].cpu().numpy(), o[2].cpu().numpy(), R, kind=okind[kind])
+                rel = oracle.error_metrics(o[3].float().cpu().numpy(), want.astype(np.float32))[0]
+                if rel > 2e-3:
+                    raise SystemExit(f"parity failure on block {N}x{K} {kind}: {rel}")
+                row[kind] = {"us_per_call": round(us, 2), "tokens_per_s": round(1e6 / us), "GBps": round(byts / us / 1e3),
+                             "frac_hbm_peak": round(byts / us / 1e3 / HBM_PEAK_GBS, 4), "rel_l2_vs_oracle": float(f"{rel:.3e}")}
+                if kind == "f16" and (N, K) == workload.LLAMA2_13B_SHAPES[0] and not args.no_cpu_baseline:
+                    W = torch.from_numpy(oracle.dequant_block_kernel_layout(o[0].cpu().numpy(), o[1].float().cpu().numpy()))
+                    us_c, n = cpu_time([(lambda x, W=W: torch.nn.functional.linear(x.float(), W), o[2].cpu())], 3.0)
+                    row["cpu_us_per_call"] = round(us_c, 1)
+                    del W
+                del bp, seq
+            c3[f"{N}x{K}x{nb}bit_R{R}"] = row
+        configs["config3_llama13b_block_alpha"] = c3
+
+        # config 5: Llama-2-70B shapes, 2 and 4 bits, 1 / 4 / 16 / 32 rows
+        c5 = {}
+        for (N, K) in workload.LLAMA2_70B_SHAPES:
+            for nb in (2, 4):
+                row = {}
+                for M in (1, 4, 16, 32):
+                    # the scalar oracle is affordable up to about a second of look-ups
+                    with_oracle = (K // 8) * N * nb * M <= (1 << 30)
+                    e, g5 = row_entry(N, K, nb, M, with_oracle)
+                    if M == 1 and (N, K, nb) == (8192, 8192, 4) and not args.no_cpu_baseline:
+                        f, _ = oracle.cpu_dense_path(g5.bW.cpu().numpy(), g5.alpha.cpu().numpy())
+                        us_c, n = cpu_time([(f, g5.x.cpu())], 6.0, max_samples=5)
+                        e["cpu_us_per_call"] = round(us_c, 1)
+                        del f
+                    del g5
+                    row[f"M{M}"] = e
+                c5[f"{N}x{K}x{nb}bit"] = row
+        configs["config5_llama70b"] = c5
+        configs["cpu_threads"] = threads
+        torch.cuda.empty_cache()
+
     # ---- config 4: full random-init Llama-2-7B decode, mixed 2/3/4-bit, batch 1 and 8 ----
     decode_res = None
     if not (args.no_decode or args.plain_only):
         from shiftaddllm_amd import decode
-        launch_mode = "eager" if graph is None else "hip-graph replay"
-        del pool, blocks, fused4, fused1, graph
+        del keep
         torch.cuda.empty_cache()
         decode_res = {}
         qc = workload.mixed_bit_config(decode.LLAMA2_7B.layers, seed=0)
@@ -475,7 +615,7 @@ def main():
     mean_bytes = step_bytes / calls_per_step
     result = {
         "metric": "lut_gemv_us_per_call_llama2_7b_3bit_batch1",
-        "value": round(us_per_call, 4),
+        "value": round(value_us, 4),
         "unit": "us/call",
         "n_gpus": 1,
         "steps": args.steps,
@@ -484,25 +624,29 @@ def main():
         "higher_is_better": False,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "f32",
+        "dtype": "f16 (fp32 accumulation)",
         "data": "synthetic",
         "config": {"workload": "llama2-7b linears, 3-bit BCQ, group 128, pow2 alpha, batch 1: "
                                f"{args.layers} blocks x 7 GEMVs per step over distinct weights "
-                               f"({step_bytes / 1e9:.3f} GB/step)",
-                   "launch": launch_mode + ", one launch per GEMV",
+                               f"({step_bytes / 1e9:.3f} GB/step); " + DATA_NOTE,
+                   "launch": launch_mode + ", one launch per GEMV; " + step_kind,
                    "calls_per_step": calls_per_step},
         "device_ms_per_step": round(dev_ms_per_step, 5),
         "achieved_GBps": round(achieved_gbs, 1),
         "frac_hbm_peak": round(achieved_gbs / HBM_PEAK_GBS, 4),
         "decode_tokens_per_s_linears_only": round(1e3 / dev_ms_per_step, 1),
+        "dependency_branches": branched,
         "roofline": {"bound": "hbm", "achieved": round(achieved_gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved_gbs / HBM_PEAK_GBS, 4), "traffic": traffic,
-                     "kernel": "lut_gemv_kernel<3, 1, 0> (nb=3, row-wise alpha)",
+                     "kernel": "lut_gemv_kernel<3, 0, 1> (nb=3, row-wise alpha, 1 row)",
                      "algorithmic_bytes_per_launch": round(mean_bytes),
-                     "avg_launch_us": round(us_per_call, 4)},
+                     "avg_launch_us": round(value_us, 4),
+                     "measured": "224 launches one after the other on one stream (graph replay), HIP events on that stream",
+                     "floors": floors},
         "cpu_baseline": cpu,
         "fused_launches": fused,
         "decode": decode_res,
+        "configs": configs,
         "parity": parity,
         "pool_build_s": round(t_pool, 2),
         "device": device_info,

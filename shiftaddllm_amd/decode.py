@@ -306,6 +306,10 @@ class LutDecoder(nn.Module):
         """Capture step() in a HIP graph (after one eager run on the capture stream,
         which also sizes the LUT-GEMM workspace of that stream)."""
         self._stream = torch.cuda.Stream()
+        # weights, caches and the step's input buffers were filled on the creating stream:
+        # without this wait the first step may read them (the token ids among them, which
+        # index the embedding table) before they have been written
+        self._stream.wait_stream(torch.cuda.current_stream())
         with torch.cuda.stream(self._stream):
             self.step()
         self._stream.synchronize()
