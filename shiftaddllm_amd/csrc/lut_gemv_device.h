@@ -194,33 +194,28 @@ __device__ __forceinline__ WindowChunk fetch_window(const Problem &p, int m0, in
     WindowChunk w;
     w.x = *(const u32x4 *)(p.x + base);
     w.other = (u32x4){0u, 0u, 0u, 0u};
-    // (the norm weight is read when the chunk is finished: a few KB shared by all
-    // workgroups, and four registers less are held until then)
     if constexpr (XF == kXGate) w.other = *(const u32x4 *)(p.gate + base);
+    if constexpr (XF == kXNorm) w.other = *(const u32x4 *)(p.norm_w + kc);
     w.kc = kc;
     w.live = k0 < p.K && rel < n_items;
     return w;
 }
 
-// Transform the chunk and park it in the window.  With a norm weight the chunk is
-// scaled by the row's reciprocal RMS and the weight; with a gate row it is multiplied
-// by silu(gate); both with the roundings of the separate fp16 operations they replace.
+// Transform the chunk and park it in the window.  With a gate row the chunk is
+// multiplied by silu(gate), with the roundings of the separate fp16 operations this
+// replaces.  With a norm weight it is multiplied by the weight only: the tables are
+// linear in their inputs, so the row's reciprocal RMS is applied to the finished sums
+// instead (flush_tile) and the reduction that yields it is not waited for here.
+// (x * weight is held as fp16: it must stay below 65504.)
 template <int MROWS, int XF>
-__device__ __forceinline__ void store_window(const Problem &p, const WindowChunk &w, const float (&rscale)[MROWS],
-                                             float *window, int tid)
+__device__ __forceinline__ void store_window(const WindowChunk &w, float *window, int tid)
 {
     u32x4 xr = w.x;
     // (opaque: the work on the fetched chunk stays here, after the sign-word requests,
     // instead of being hoisted to where it would have to wait for the chunk first)
     asm volatile("" : "+v"(xr.x), "+v"(xr.y), "+v"(xr.z), "+v"(xr.w));
     if constexpr (XF != kXNone) {
-        constexpr int kSlots = kWindowSlots / MROWS;
-        const int row = tid / (kTables * kSlots);
-        float rs = rscale[0];
-#pragma unroll
-        for (int r = 1; r < MROWS; ++r) rs = row == r ? rscale[r] : rs;
-        u32x4 other = w.other;
-        if constexpr (XF == kXNorm) other = *(const u32x4 *)(p.norm_w + w.kc);
+        const u32x4 other = w.other;
         const uint32_t a[4] = {xr.x, xr.y, xr.z, xr.w};
         const uint32_t b[4] = {other.x, other.y, other.z, other.w};
         uint32_t o[4];
@@ -234,7 +229,7 @@ __device__ __forceinline__ void store_window(const Problem &p, const WindowChunk
                 if constexpr (XF == kXGate)
                     v[hh] = half_bits_to_float(float_to_half_bits(__fdividef(bv, 1.0f + __expf(-bv)))) * xv;
                 else
-                    v[hh] = half_bits_to_float(float_to_half_bits(xv * rs)) * bv;
+                    v[hh] = xv * bv;
             }
             o[j] = float_to_half_bits(v[0]) | (float_to_half_bits(v[1]) << 16);
         }
@@ -364,6 +359,29 @@ __device__ __forceinline__ float swizzle_xor(float v)
     return __builtin_bit_cast(float, __builtin_amdgcn_ds_swizzle(__builtin_bit_cast(int, v), (XOR << 10) | 0x1f));
 }
 
+// The value of another lane of the same row of 16, by a data-parallel-primitive move.
+template <int CTRL>
+__device__ __forceinline__ float dpp_move(float v)
+{
+    const int vi = __builtin_bit_cast(int, v);
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(vi, vi, CTRL, 0xf, 0xf, false));
+}
+
+// Sum over the 64 lanes of a wave, on the vector ALU: xor 1 and 2 inside quads, then the
+// mirrored quad and the mirrored half of each row of 16, then the four rows.
+__device__ __forceinline__ float wave_sum(float v)
+{
+    v += dpp_move<0xb1>(v);   // quad_perm [1,0,3,2]
+    v += dpp_move<0x4e>(v);   // quad_perm [2,3,0,1]
+    v += dpp_move<0x141>(v);  // row_half_mirror
+    v += dpp_move<0x140>(v);  // row_mirror
+    const int vi = __builtin_bit_cast(int, v);
+    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(vi, 0)) +
+           __builtin_bit_cast(float, __builtin_amdgcn_readlane(vi, 16)) +
+           __builtin_bit_cast(float, __builtin_amdgcn_readlane(vi, 32)) +
+           __builtin_bit_cast(float, __builtin_amdgcn_readlane(vi, 48));
+}
+
 // Reduce-scatter of the 8 kw-lanes of a quad: each lane comes in with its partial
 // sums of 4 outputs and leaves with the complete sum of output
 // i = 2*(kw>>2 & 1) + (kw>>1 & 1); lanes kw and kw^1 hold the same value.
@@ -491,44 +509,45 @@ __device__ __forceinline__ void gemv_range(const Problem &p, int range, int mchu
         }
         fetch_out(tile);
     };
-    // Also once, after that: finish the reciprocal RMS and park the first window.
+    // Also once, after that: park the first window and, with a fused RMSNorm, leave each
+    // wave's share of the rows' sums of squares in LDS.  The reciprocal RMS is formed
+    // from those behind the barrier and is first needed when sums are handed over.
     auto first_window = [&]() {
         if constexpr (XF == kXNorm) {
-            float ss[MROWS];
+            static_assert(XF != kXNorm || !is_staged(MODE), "the per-wave sums live in the alpha staging area");
 #pragma unroll
             for (int r = 0; r < MROWS; ++r) {
-                ss[r] = 0.0f;
+                float ss = 0.0f;
                 auto add_chunk = [&](const u32x4 &v) {
                     const uint32_t w4[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll
                     for (int j = 0; j < 4; ++j) {
                         const float lo = half_bits_to_float(w4[j] & 0xffffu), hi = half_bits_to_float(w4[j] >> 16);
-                        ss[r] = fmaf(lo, lo, fmaf(hi, hi, ss[r]));
+                        ss = fmaf(lo, lo, fmaf(hi, hi, ss));
                     }
                 };
 #pragma unroll
                 for (int u = 0; u < kNormChunks; ++u)
                     if (tid + kThreads * u < p.K / 8) add_chunk(nx[r][u]);
-                for (int c = tid + kThreads * kNormChunks; c < p.K / 8; c += kThreads)  // K > 16384
+                for (int c = tid + kThreads * kNormChunks; c < p.K / 8; c += kThreads)  // K > 8192
                     add_chunk(*(const u32x4 *)(xrow[r] + 8 * c));
-#pragma unroll
-                for (int off = 32; off > 0; off >>= 1) ss[r] += __shfl_xor(ss[r], off);
-                if (lane == 0) lut[wave * MROWS + r] = ss[r];
+                ss = wave_sum(ss);
+                if (lane == 0) stage[wave * MROWS + r] = ss;
             }
-            __syncthreads();
+        }
+        store_window<MROWS, XF>(w0, window, tid);
+        // (without a transform the first build does not read the window, and the barrier
+        // that follows that build publishes the window as well)
+        if constexpr (XF != kXNone) __syncthreads();
+        if constexpr (XF == kXNorm) {
 #pragma unroll
             for (int r = 0; r < MROWS; ++r) {
                 float t = 0.0f;
 #pragma unroll
-                for (int w = 0; w < kWaves; ++w) t += lut[w * MROWS + r];
+                for (int w = 0; w < kWaves; ++w) t += stage[w * MROWS + r];
                 rscale[r] = rsqrtf(t / (float)p.K + p.norm_eps);
             }
-            // (the tables are built over the same LDS words: the barrier below orders that)
         }
-        store_window<MROWS, XF>(p, w0, rscale, window, tid);
-        // (without a transform the first build does not read the window, and the barrier
-        // that follows that build publishes the window as well)
-        if constexpr (XF != kXNone) __syncthreads();
     };
 
     // ---- hand a tile's complete K-slice over ---------------------------------------
@@ -543,7 +562,8 @@ __device__ __forceinline__ void gemv_range(const Problem &p, int range, int mchu
         const bool owner = (kw2 & 1) == 0;
 #pragma unroll
         for (int r = 0; r < MROWS; ++r) {
-            const float v = reduce_scatter_kw(acc[r], kw2);
+            float v = reduce_scatter_kw(acc[r], kw2);
+            if constexpr (XF == kXNorm) v *= rscale[r];
 #pragma unroll
             for (int i = 0; i < 4; ++i) acc[r][i] = 0.0f;
             const int m = m0 + r;
@@ -587,7 +607,7 @@ __device__ __forceinline__ void gemv_range(const Problem &p, int range, int mchu
             // a window's items only occur beyond half a billion weights per call, and a
             // conditional load in flight would make every later wait conservative.
             const WindowChunk w = fetch_window<MROWS, XF>(p, m0, set0, rel, n_items, tid);
-            store_window<MROWS, XF>(p, w, rscale, window, tid);
+            store_window<MROWS, XF>(w, window, tid);
             __syncthreads();
         }
 #pragma unroll
