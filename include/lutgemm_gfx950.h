@@ -220,7 +220,7 @@ int lutgemm_release_workspaces(void);
  * folded in (no counterpart in the reference, whose modules run them as
  * separate framework kernels).  Up to LUTGEMM_MAX_GROUP problems per launch.
  *   norm_weight_f16 : NULL, or fp16 [K]: the GEMV input is
- *                     fp16(fp16(x * rsqrt(mean(x^2) + norm_eps)) * norm_weight)
+ *                     x * rsqrt(mean(x^2) + norm_eps) * norm_weight
  *                     per row of x (RMSNorm), formed inside the kernel;
  *   gate_f16        : NULL, or fp16 [M][K]: the GEMV input is
  *                     fp16(fp16(silu(gate)) * x)  (SwiGLU);
@@ -233,6 +233,27 @@ int lutgemm_release_workspaces(void);
  * look-up kernel, whatever M (with several rows a separate transform kernel in
  * front of a plain call is faster); overwriting problems with several rows take
  * the matrix-core kernel like plain ones.
+ *
+ * With norm_weight_f16 the kernel multiplies x by the weight first (x * weight is
+ * held as fp16 and must stay below 65504) and applies rsqrt(mean(x^2) + norm_eps)
+ * to the finished sums, which is the same product.
+ *
+ * RMSNorm split over two launches, for a residual stream that one GEMV completes
+ * and the next reads normalised (either look-up or matrix-core kernel, any M):
+ *   the completing problem (out = residual, accumulated into) names
+ *     next_norm_weight_f16 : fp16 [N], the weight of the norm that follows,
+ *     next_input_f16       : fp16 [M][N], receives fp16(out * next_norm_weight),
+ *     sumsq_out_f32        : float [M][N/32], ZERO before the call (N % 32 == 0):
+ *                            receives, spread over a row's slots, the sum of the
+ *                            squares of the row's final outputs;
+ *   the consuming problem takes x_f16 = that next_input, K = that N, and
+ *     sumsq_in_f32 / sumsq_in_slots : that array (16-byte aligned) and its N/32 slots per row:
+ *                            y = rsqrt(sum(slots) / K + norm_eps) * W x.
+ *   All five may be NULL / 0; next_norm_weight and next_input come together;
+ *   sumsq_in excludes norm_weight_f16.  Which slot receives which columns is
+ *   unspecified; a slot normally receives one float add (two when outputs of a
+ *   32-column run were completed by different workgroups), so the sums are
+ *   reproducible from run to run.
  */
 typedef struct lutgemm_fused_problem {
     const uint32_t *bW;
@@ -244,6 +265,11 @@ typedef struct lutgemm_fused_problem {
     const void *norm_weight_f16;
     const void *gate_f16;
     float norm_eps;
+    const void *next_norm_weight_f16;
+    void *next_input_f16;
+    float *sumsq_out_f32;
+    const float *sumsq_in_f32;
+    int sumsq_in_slots;
 } lutgemm_fused_problem;
 
 int lutgemm_gemv_rowwise_f16_fused(int count, const lutgemm_fused_problem *problems, void *stream);

@@ -16,7 +16,28 @@ hipError_t launch_nb(const Problem &p, int mt, hipStream_t stream)
     return hipGetLastError();
 }
 
+template <int NB>
+hipError_t launch_fused_nb(const Problem &p, int mt, hipStream_t stream)
+{
+    const dim3 grid((unsigned)p.n_blocks), block(kMfmaThreads);
+    if (mt == 2)
+        hipLaunchKernelGGL((lut_gemm_mfma_fused_kernel<NB, 2>), grid, block, 0, stream, p);
+    else
+        hipLaunchKernelGGL((lut_gemm_mfma_fused_kernel<NB, 1>), grid, block, 0, stream, p);
+    return hipGetLastError();
+}
+
 }  // namespace
+
+hipError_t launch_mfma_fused(const Problem &p, int mt, hipStream_t stream)
+{
+    switch (p.nb) {
+    case 1: return launch_fused_nb<1>(p, mt, stream);
+    case 2: return launch_fused_nb<2>(p, mt, stream);
+    case 3: return launch_fused_nb<3>(p, mt, stream);
+    default: return launch_fused_nb<4>(p, mt, stream);
+    }
+}
 
 hipError_t launch_mfma(const Problem &p, int mt, hipStream_t stream)
 {
@@ -30,7 +51,7 @@ hipError_t launch_mfma(const Problem &p, int mt, hipStream_t stream)
 
 hipError_t launch_mfma_group(const Group &g, int mt, int blocks, hipStream_t stream)
 {
-    const dim3 grid((unsigned)blocks), block(kMfmaThreads);
+    const dim3 grid((unsigned)blocks, (unsigned)g.count), block(kMfmaThreads);
     if (mt == 2)
         hipLaunchKernelGGL((lut_gemm_mfma_group_kernel<2>), grid, block, 0, stream, g);
     else

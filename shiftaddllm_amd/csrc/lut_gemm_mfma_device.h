@@ -48,7 +48,9 @@ constexpr int kMfmaTileCols = 64;     // outputs per workgroup
 constexpr int kMfmaStepK = 128;
 constexpr int kRedRow = 65;           // the final reduction's LDS rows, padded against bank conflicts
 template <int MT>
-constexpr int kMfmaLdsBytes = kMfmaWaves * 16 * MT * kRedRow * 4;
+constexpr int kMfmaRedBytes = kMfmaWaves * 16 * MT * kRedRow * 4;
+template <int MT>
+constexpr int kMfmaLdsBytes = kMfmaRedBytes<MT> + 16 * MT * 4;
 
 // Operands of one K-step of a wave: per bit plane word kb of 4 outputs and their
 // alphas; per 16-row tile the lane's 32 activations.
@@ -96,8 +98,10 @@ __device__ __forceinline__ f16x8 expand_signs(uint32_t w, int beta, uint32_t alp
     return __builtin_bit_cast(f16x8, r);
 }
 
-// xs: kMfmaLdsBytes<MT> bytes of LDS for the final reduction.
-template <int NB, int MT>
+// xs: kMfmaLdsBytes<MT> bytes of LDS for the final reduction (and, behind them, the
+// reciprocal RMS of the tile's rows).
+// EXTRA: the launch honours the split-RMSNorm fields of the problem (next_in, sumsq_*).
+template <int NB, int MT, bool EXTRA = false>
 __device__ __forceinline__ void mfma_tile(const Problem &p, int local_block, char *xs)
 {
     const int tid = threadIdx.x;
@@ -122,6 +126,44 @@ __device__ __forceinline__ void mfma_tile(const Problem &p, int local_block, cha
     const __half *xlane[MT];
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) xlane[mt] = p.x + (size_t)min(m0 + 16 * mt + li, p.M - 1) * p.K + 32 * kb;
+
+    // split RMSNorm, consuming side: wave w sums the slots of rows w, w + 8, ... and leaves
+    // their reciprocal RMS in LDS for the hand-over
+    // The slots are requested here, ahead of everything else, and summed once the first
+    // step's operands have been requested behind them (see the main loop): loads return in
+    // order, so that wait is for the slots alone.
+    float *row_scale = (float *)(xs + kMfmaRedBytes<MT>);
+    typedef float f32x4v __attribute__((ext_vector_type(4)));
+    constexpr int kScaleRows = 2 * MT;  // rows per wave
+    bool scaled = false;
+    [[maybe_unused]] f32x4v slot4[kScaleRows];
+    // (the wave index as a scalar, so that the rows' addresses are a scalar base plus one lane offset)
+    const int wave_s = __builtin_amdgcn_readfirstlane(wave);
+    if constexpr (EXTRA) {
+        scaled = p.sumsq_in != nullptr;
+        if (scaled) {
+            // one 16-byte request per row and lane: 256 slots, inputs up to 8192 (slots = K / 32
+            // and K % 128 == 0 on this path)
+            const int quads = p.sumsq_slots >> 2;
+#pragma unroll
+            for (int i = 0; i < kScaleRows; ++i) {
+                const float *slots = p.sumsq_in + (size_t)min(m0 + wave_s + kMfmaWaves * i, p.M - 1) * p.sumsq_slots;
+                slot4[i] = *((const f32x4v *)slots + min(lane, quads - 1));
+            }
+        }
+    }
+    auto row_scales = [&]() {
+        const int quads = p.sumsq_slots >> 2;
+#pragma unroll
+        for (int i = 0; i < kScaleRows; ++i) {
+            const int row = wave_s + kMfmaWaves * i;
+            const float *slots = p.sumsq_in + (size_t)min(m0 + row, p.M - 1) * p.sumsq_slots;
+            float t = lane < quads ? (slot4[i].x + slot4[i].y) + (slot4[i].z + slot4[i].w) : 0.0f;
+            for (int c = 4 * 64 + lane; c < p.sumsq_slots; c += 64) t += slots[c];  // inputs beyond 8192
+            t = wave_sum(t);
+            if (lane == 0) row_scale[row] = rsqrtf(t / (float)p.K + p.norm_eps);
+        }
+    };
 
     f32x4 acc[4][MT];
 #pragma unroll
@@ -185,12 +227,16 @@ __device__ __forceinline__ void mfma_tile(const Problem &p, int local_block, cha
         mfma_load<NB, MT>(opA, p, min(s, last_step), kb, wcol4, xlane);
         __builtin_amdgcn_sched_barrier(0);
         if (!first) compute(opB);
+        if constexpr (EXTRA)
+            if (first && scaled) row_scales();
         __builtin_amdgcn_sched_barrier(0);
         mfma_load<NB, MT>(opB, p, min(s + kMfmaWaves, last_step), kb, wcol4, xlane);
         __builtin_amdgcn_sched_barrier(0);
         compute(opA);
     }
     if (n_steps > 0 && (n_steps & 1) == 0) compute(opB);
+    if constexpr (EXTRA)
+        if (n_steps == 0 && scaled) row_scales();  // (a wave without steps still owes its rows)
 
     // ---- the 8 waves' accumulators meet in LDS -----------------------------------
     // red[wave][j = (e*MT + mt)*4 + r][lane], rows padded to 65 words so that the
@@ -211,6 +257,9 @@ __device__ __forceinline__ void mfma_tile(const Problem &p, int local_block, cha
     const int n = n_base + nl;
     const int src_lane = (nl >> 4) * 16;            // kb of the column; + li of the row below
     const int src_j = (nl & 3) * MT * 4 + ((nl >> 2) & 3);  // e and r of the column; + mt*4 of the row
+    [[maybe_unused]] float next_w = 0.0f;
+    if constexpr (EXTRA)
+        if (p.next_w) next_w = __half2float(p.next_w[min(n, p.N - 1)]);
     float val[2 * MT];
     Contribution contrib[2 * MT];
     unsigned long long old[2 * MT];
@@ -221,6 +270,7 @@ __device__ __forceinline__ void mfma_tile(const Problem &p, int local_block, cha
         float v = 0.0f;
 #pragma unroll
         for (int w = 0; w < kMfmaWaves; ++w) v += red[(w * (16 * MT) + j) * kRedRow + sl];
+        if (scaled) v *= row_scale[ml];
         val[i] = v;
         old[i] = 0;
         contrib[i] = Contribution{0ull, 0ull};
@@ -236,16 +286,28 @@ __device__ __forceinline__ void mfma_tile(const Problem &p, int local_block, cha
 #pragma unroll
     for (int i = 0; i < 2 * MT; ++i) {
         const int m = m0 + (tid >> 6) + 8 * i;
-        if (m >= p.M || n >= p.N) continue;
-        __half *dst = p.out + (size_t)m * p.N + n;
-        if (p.ksplit == 1) {
-            *dst = __float2half_rn((p.overwrite ? 0.0f : __half2float(*dst)) + val[i]);
-            continue;
+        [[maybe_unused]] float sq = 0.0f;  // square of the output this thread completed
+        if (m < p.M && n < p.N && (p.ksplit == 1 || (int)(old[i] >> 56) == p.ksplit - 1)) {
+            __half *dst = p.out + (size_t)m * p.N + n;
+            const float y = p.ksplit == 1 ? val[i] : fixed_total((old[i] | contrib[i].flags) + contrib[i].add, p.ksplit);
+            const __half y16 = __float2half_rn((p.overwrite ? 0.0f : __half2float(*dst)) + y);
+            *dst = y16;
+            if (p.ksplit > 1)
+                __hip_atomic_store(p.accum + (size_t)m * p.N + n, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if constexpr (EXTRA) {
+                const float yf = __half2float(y16);
+                sq = yf * yf;
+                if (p.next_in) p.next_in[(size_t)m * p.N + n] = __float2half_rn(yf * next_w);
+            }
         }
-        if ((int)(old[i] >> 56) != p.ksplit - 1) continue;
-        const float y = fixed_total((old[i] | contrib[i].flags) + contrib[i].add, p.ksplit);
-        *dst = __float2half_rn((p.overwrite ? 0.0f : __half2float(*dst)) + y);
-        __hip_atomic_store(p.accum + (size_t)m * p.N + n, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if constexpr (EXTRA) {
+            // the wave's 64 columns of row m: one add into the first of their two slots
+            if (p.sumsq_out) {
+                const float s = wave_sum(sq);
+                if (lane == 0 && m < p.M && s != 0.0f)
+                    unsafeAtomicAdd(p.sumsq_out + (size_t)m * (p.N / 32) + n_base / 32, s);
+            }
+        }
     }
 }
 
@@ -256,22 +318,30 @@ __global__ void __launch_bounds__(kMfmaThreads) lut_gemm_mfma_kernel(const Probl
     mfma_tile<NB, MT>(p, (int)blockIdx.x, xs);
 }
 
-// Several problems in one launch (flat 1-D grid); bit widths may differ.
+// One problem with the split-RMSNorm fields honoured.
+template <int NB, int MT>
+__global__ void __launch_bounds__(kMfmaThreads) lut_gemm_mfma_fused_kernel(const Problem p)
+{
+    __shared__ __attribute__((aligned(16))) char xs[kMfmaLdsBytes<MT>];
+    mfma_tile<NB, MT, true>(p, (int)blockIdx.x, xs);
+}
+
+// Several problems in one launch; bit widths may differ.
 template <int MT>
 __global__ void __launch_bounds__(kMfmaThreads) lut_gemm_mfma_group_kernel(const Group g)
 {
     __shared__ __attribute__((aligned(16))) char xs[kMfmaLdsBytes<MT>];
+    // grid = (workgroups of the largest problem, problems)
+    // (through the constant address space, which the kernel arguments live in: the fields are
+    // then scalar loads that may be repeated at will instead of values to keep in registers)
+    const Problem &p = *(const Problem *)((const __attribute__((address_space(4))) Problem *)&g.p[0] + blockIdx.y);
     const int b = blockIdx.x;
-    int pi = 0;
-#pragma unroll
-    for (int i = 1; i < kMaxGroup; ++i)
-        if (i < g.count && b >= g.p[i].block_begin) pi = i;
-    const Problem &p = g.p[pi];
+    if (b >= p.n_blocks) return;
     switch (p.nb) {
-    case 1: mfma_tile<1, MT>(p, b - p.block_begin, xs); break;
-    case 2: mfma_tile<2, MT>(p, b - p.block_begin, xs); break;
-    case 3: mfma_tile<3, MT>(p, b - p.block_begin, xs); break;
-    default: mfma_tile<4, MT>(p, b - p.block_begin, xs); break;
+    case 1: mfma_tile<1, MT, true>(p, b, xs); break;
+    case 2: mfma_tile<2, MT, true>(p, b, xs); break;
+    case 3: mfma_tile<3, MT, true>(p, b, xs); break;
+    default: mfma_tile<4, MT, true>(p, b, xs); break;
     }
 }
 

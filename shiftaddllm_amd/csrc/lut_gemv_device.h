@@ -359,29 +359,6 @@ __device__ __forceinline__ float swizzle_xor(float v)
     return __builtin_bit_cast(float, __builtin_amdgcn_ds_swizzle(__builtin_bit_cast(int, v), (XOR << 10) | 0x1f));
 }
 
-// The value of another lane of the same row of 16, by a data-parallel-primitive move.
-template <int CTRL>
-__device__ __forceinline__ float dpp_move(float v)
-{
-    const int vi = __builtin_bit_cast(int, v);
-    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(vi, vi, CTRL, 0xf, 0xf, false));
-}
-
-// Sum over the 64 lanes of a wave, on the vector ALU: xor 1 and 2 inside quads, then the
-// mirrored quad and the mirrored half of each row of 16, then the four rows.
-__device__ __forceinline__ float wave_sum(float v)
-{
-    v += dpp_move<0xb1>(v);   // quad_perm [1,0,3,2]
-    v += dpp_move<0x4e>(v);   // quad_perm [2,3,0,1]
-    v += dpp_move<0x141>(v);  // row_half_mirror
-    v += dpp_move<0x140>(v);  // row_mirror
-    const int vi = __builtin_bit_cast(int, v);
-    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(vi, 0)) +
-           __builtin_bit_cast(float, __builtin_amdgcn_readlane(vi, 16)) +
-           __builtin_bit_cast(float, __builtin_amdgcn_readlane(vi, 32)) +
-           __builtin_bit_cast(float, __builtin_amdgcn_readlane(vi, 48));
-}
-
 // Reduce-scatter of the 8 kw-lanes of a quad: each lane comes in with its partial
 // sums of 4 outputs and leaves with the complete sum of output
 // i = 2*(kw>>2 & 1) + (kw>>1 & 1); lanes kw and kw^1 hold the same value.
@@ -403,9 +380,11 @@ __device__ __forceinline__ float reduce_scatter_kw(const float (&acc)[4], int kw
 // `mchunk` (activation rows mchunk*MROWS .. +MROWS-1).  The sign words of an item
 // are loaded once and used for all MROWS rows; tables are built per (item, row)
 // and double buffered.
-template <int NB, int MODE, int MROWS, int XF = kXNone>
+// EXTRA: the launch honours the split-RMSNorm fields of the problem (next_in, sumsq_*).
+template <int NB, int MODE, int MROWS, int XF = kXNone, bool EXTRA = false>
 __device__ __forceinline__ void gemv_range(const Problem &p, int range, int mchunk, float *lut)
 {
+    static_assert(!(EXTRA || XF == kXNorm) || !is_staged(MODE), "the per-wave sums live in the alpha staging area");
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = tid >> 6;
@@ -461,11 +440,12 @@ __device__ __forceinline__ void gemv_range(const Problem &p, int range, int mchu
     const int set0 = set, n_items = rem;
     float *window = stage + kStageDwords;
     const WindowChunk w0 = fetch_window<MROWS, XF>(p, m0, set0, 0, n_items, tid);
+    constexpr bool kDirectFirst = XF == kXNone;
     // Without an input transform the tables of the first item (row 0) are built straight
     // from a second request for this thread's own chunk, so that nothing but that chunk
     // stands between the start of the kernel and the first table.
     u32x4 x0 = (u32x4){0u, 0u, 0u, 0u};
-    if constexpr (XF == kXNone) {
+    if constexpr (kDirectFirst) {
         const int k0 = (set0 * kTables + tb) * 8;
         x0 = *(const u32x4 *)(xrow[0] + min(k0, p.K - 8));
     }
@@ -481,6 +461,20 @@ __device__ __forceinline__ void gemv_range(const Problem &p, int range, int mchu
             for (int u = 0; u < kNormChunks; ++u)
                 nx[r][u] = *(const u32x4 *)(xrow[r] + 8 * min(tid + kThreads * u, p.K / 8 - 1));
     }
+    // split RMSNorm, consuming side: this thread's share of the rows' sums of squares
+    float slot_sum[MROWS];
+#pragma unroll
+    for (int r = 0; r < MROWS; ++r) slot_sum[r] = 0.0f;
+    if constexpr (EXTRA) {
+        // one clamped, unconditional request per row here (a loop would wait for each load,
+        // and with it for everything requested above); more than kThreads slots are rare
+        // and fetched in first_window
+        if (p.sumsq_in) {
+#pragma unroll
+            for (int r = 0; r < MROWS; ++r)
+                slot_sum[r] = p.sumsq_in[(size_t)min(m0 + r, p.M - 1) * p.sumsq_slots + min(tid, p.sumsq_slots - 1)];
+        }
+    }
     // the caller's output, needed only by whoever completes a sum: fetched early,
     // off the critical path (again whenever the range moves on to another tile)
     unsigned short out_prev[MROWS];
@@ -492,9 +486,6 @@ __device__ __forceinline__ void gemv_range(const Problem &p, int range, int mchu
     };
     __builtin_amdgcn_sched_barrier(0);  // keep these requests ahead of the sign words
 
-    float rscale[MROWS];
-#pragma unroll
-    for (int r = 0; r < MROWS; ++r) rscale[r] = 1.0f;
     // Runs once, after the first operand loads have been issued: everything the look-ups
     // and the hand-over need but the first requests did not.
     auto late_setup = [&]() {
@@ -514,7 +505,6 @@ __device__ __forceinline__ void gemv_range(const Problem &p, int range, int mchu
     // from those behind the barrier and is first needed when sums are handed over.
     auto first_window = [&]() {
         if constexpr (XF == kXNorm) {
-            static_assert(XF != kXNorm || !is_staged(MODE), "the per-wave sums live in the alpha staging area");
 #pragma unroll
             for (int r = 0; r < MROWS; ++r) {
                 float ss = 0.0f;
@@ -535,19 +525,33 @@ __device__ __forceinline__ void gemv_range(const Problem &p, int range, int mchu
                 if (lane == 0) stage[wave * MROWS + r] = ss;
             }
         }
+        if constexpr (EXTRA) {
+            if (p.sumsq_in) {
+#pragma unroll
+                for (int r = 0; r < MROWS; ++r) {
+                    // (opaque: the work on the fetched value stays here, behind the sign-word
+                    // requests, instead of being hoisted to where it would have to wait first)
+                    asm volatile("" : "+v"(slot_sum[r]));
+                    float v = tid < p.sumsq_slots ? slot_sum[r] : 0.0f;
+                    for (int c = tid + kThreads; c < p.sumsq_slots; c += kThreads)
+                        v += p.sumsq_in[(size_t)min(m0 + r, p.M - 1) * p.sumsq_slots + c];
+                    const float s = wave_sum(v);
+                    if (lane == 0) stage[wave * MROWS + r] = s;
+                }
+            }
+        }
         store_window<MROWS, XF>(w0, window, tid);
         // (without a transform the first build does not read the window, and the barrier
         // that follows that build publishes the window as well)
-        if constexpr (XF != kXNone) __syncthreads();
-        if constexpr (XF == kXNorm) {
+        if constexpr (!kDirectFirst) __syncthreads();
+    };
+    // A row's reciprocal RMS from the per-wave sums (any time after the first barrier
+    // that follows first_window; formed where it is used rather than kept in a register).
+    auto row_scale = [&](int r) {
+        float t = 0.0f;
 #pragma unroll
-            for (int r = 0; r < MROWS; ++r) {
-                float t = 0.0f;
-#pragma unroll
-                for (int w = 0; w < kWaves; ++w) t += stage[w * MROWS + r];
-                rscale[r] = rsqrtf(t / (float)p.K + p.norm_eps);
-            }
-        }
+        for (int w = 0; w < kWaves; ++w) t += stage[w * MROWS + r];
+        return rsqrtf(t / (float)p.K + p.norm_eps);
     };
 
     // ---- hand a tile's complete K-slice over ---------------------------------------
@@ -560,18 +564,38 @@ __device__ __forceinline__ void gemv_range(const Problem &p, int range, int mchu
         asm volatile("" : "+v"(kw2));  // (opaque: see own_col_of)
         const int n = t * kTileCols + own_col_of(kw2);
         const bool owner = (kw2 & 1) == 0;
+        bool scaled = XF == kXNorm;
+        if constexpr (EXTRA) scaled = scaled || p.sumsq_in != nullptr;
+        // the next norm's weight for this lane's column: requested here, used once the
+        // sums are complete
+        [[maybe_unused]] unsigned short next_w_bits = 0;
+        if constexpr (EXTRA)
+            if (p.next_w) next_w_bits = *((const unsigned short *)p.next_w + min(n, p.N - 1));
+        [[maybe_unused]] float sq[MROWS];  // squares of the outputs this lane completed
+        // An output is complete: round it, write it and, with a split RMSNorm, its product
+        // with the next norm's weight beside it.
+        auto complete = [&](int r, __half *dst, float y) {
+            const __half y16 = __float2half_rn(y);
+            *dst = y16;
+            if constexpr (EXTRA) {
+                const float yf = __half2float(y16);
+                sq[r] = yf * yf;
+                if (p.next_in) p.next_in[dst - p.out] = __float2half_rn(yf * half_bits_to_float(next_w_bits));
+            }
+        };
 #pragma unroll
         for (int r = 0; r < MROWS; ++r) {
             float v = reduce_scatter_kw(acc[r], kw2);
-            if constexpr (XF == kXNorm) v *= rscale[r];
+            if (scaled) v *= row_scale(r);
 #pragma unroll
             for (int i = 0; i < 4; ++i) acc[r][i] = 0.0f;
+            if constexpr (EXTRA) sq[r] = 0.0f;
             const int m = m0 + r;
             if (!owner || n >= p.N || m >= p.M) continue;
             __half *dst = p.out + (size_t)m * p.N + n;
             const float prev = p.overwrite ? 0.0f : half_bits_to_float(out_prev[r]);
             if (count == 1 && p.finish == kFinishInline) {
-                *dst = __float2half_rn(prev + v);
+                complete(r, dst, prev + v);
                 continue;
             }
             unsigned long long *word = p.accum + (size_t)m * p.N + n;
@@ -585,8 +609,21 @@ __device__ __forceinline__ void gemv_range(const Problem &p, int range, int mchu
                 __hip_atomic_fetch_add(word, c.add, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             if ((int)(old >> 56) != count - 1) continue;
             // this contribution completed the sum
-            *dst = __float2half_rn(prev + fixed_total((old | c.flags) + c.add, count));
+            complete(r, dst, prev + fixed_total((old | c.flags) + c.add, count));
             __hip_atomic_store(word, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        if constexpr (EXTRA) {
+            // The wave's 32 columns are one slot of the row's sums of squares.  Normally one
+            // wave completes all 32 and the slot receives a single add; when completions
+            // are split between workgroups it receives one add from each.
+            if (p.sumsq_out) {
+#pragma unroll
+                for (int r = 0; r < MROWS; ++r) {
+                    const float s = wave_sum(sq[r]);
+                    if (lane == 0 && s != 0.0f)
+                        unsafeAtomicAdd(p.sumsq_out + (size_t)(m0 + r) * (p.N / kWaveCols) + t * kWaves + wave, s);
+                }
+            }
         }
     };
 
@@ -613,7 +650,7 @@ __device__ __forceinline__ void gemv_range(const Problem &p, int range, int mchu
 #pragma unroll
         for (int r = 0; r < MROWS; ++r) {
             u32x4 xr = x0;
-            if (XF != kXNone || r > 0 || rel > 0) {
+            if (!kDirectFirst || r > 0 || rel > 0) {
                 xr = *(const u32x4 *)(window + 4 * ((r * kSlots + slot) * kTables + tb));
             } else {
                 // (opaque, so that the chunk is not waited for before it is needed)
@@ -690,27 +727,27 @@ lut_gemv_kernel(const Problem p)
     gemv_range<NB, MODE, MROWS>(p, (int)blockIdx.x, (int)blockIdx.y, lut);  // grid = (ranges, row chunks)
 }
 
-// Several row-wise problems in one launch (flat 1-D grid).  Bit widths may
-// differ between the problems of a group.
+// Several row-wise problems in one launch.  Bit widths may differ between the
+// problems of a group.
 // XF: the input transform shared by all problems of the launch.
 template <int XF>
 __global__ void __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4, 4)))
 lut_gemv_group_kernel(const Group g)
 {
     __shared__ __attribute__((aligned(16))) float lut[kLutDwords + kStageDwords + kWindowDwords];
-    const int b = blockIdx.x;
-    int pi = 0;
-#pragma unroll
-    for (int i = 1; i < kMaxGroup; ++i)
-        if (i < g.count && b >= g.p[i].block_begin) pi = i;
-    const Problem &p = g.p[pi];
+    // grid = (workgroups of the largest problem, problems): the problem is known from the
+    // dispatch, so its fields are one scalar-load round trip away like a lone problem's
+    // (through the constant address space, which the kernel arguments live in: the fields are
+    // then scalar loads that may be repeated at will instead of values to keep in registers)
+    const Problem &p = *(const Problem *)((const __attribute__((address_space(4))) Problem *)&g.p[0] + blockIdx.y);
+    if ((int)blockIdx.x >= p.n_blocks) return;
     int range, m;
-    decode_block(p, b - p.block_begin, range, m);
+    decode_block(p, (int)blockIdx.x, range, m);
     switch (p.nb) {
-    case 1: gemv_range<1, kRowF16, 1, XF>(p, range, m, lut); break;
-    case 2: gemv_range<2, kRowF16, 1, XF>(p, range, m, lut); break;
-    case 3: gemv_range<3, kRowF16, 1, XF>(p, range, m, lut); break;
-    default: gemv_range<4, kRowF16, 1, XF>(p, range, m, lut); break;
+    case 1: gemv_range<1, kRowF16, 1, XF, true>(p, range, m, lut); break;
+    case 2: gemv_range<2, kRowF16, 1, XF, true>(p, range, m, lut); break;
+    case 3: gemv_range<3, kRowF16, 1, XF, true>(p, range, m, lut); break;
+    default: gemv_range<4, kRowF16, 1, XF, true>(p, range, m, lut); break;
     }
 }
 

@@ -7,7 +7,7 @@ namespace lutgemm {
 
 hipError_t launch_gemv_group(const Group &g, int xform, int blocks, hipStream_t stream)
 {
-    const dim3 grid((unsigned)blocks), block(kThreads);
+    const dim3 grid((unsigned)blocks, (unsigned)g.count), block(kThreads);
     if (xform == kXNorm)
         hipLaunchKernelGGL((lut_gemv_group_kernel<kXNorm>), grid, block, 0, stream, g);
     else if (xform == kXGate)

@@ -103,40 +103,54 @@ __device__ __forceinline__ int fast_div(int n, const Divisor &d)
     return (int)__umulhi((uint32_t)(2 * n) >> d.shift, d.magic);
 }
 
+// Field order: a kernel fetches its arguments a cache line at a time, on demand, and
+// each line touched for the first time before the sign words are requested is a round
+// trip on the start-up path.  What the kernels need to issue their first loads comes
+// first (two 64-byte lines), what the hand-over of finished sums needs comes last.
 struct Problem {
+    // ---- needed to request the first operands -----------------------------------------
     const uint32_t *W;
     const void *alpha;
-    const __half *qbias;
     const __half *x;
-    __half *out;
-    unsigned long long *accum;  // [M][N] fixed-point words, zero between launches
+    const float *sumsq_in;  // split RMSNorm, consuming side: [M][sumsq_slots] (see below)
     int N, K, M;
     int kwords;          // K / 32
     int nsets;           // look-up kernel: ceil(kwords / 8); matrix-core kernel: K-steps
     int n_tiles;
     int group_words;     // row-wise / uniform: words per alpha group
+    int nb;
     Divisor by_group_words;  // row / group_words
     Divisor by_nsets;        // item / nsets
     Divisor by_items;        // item / items_per_wg
-    int R;               // block modes: row groups
-    int rows_per_group;  // block modes: N / R
-    int nb;
-    int block_begin;     // grouped launches: first flat workgroup index of this problem
-    int mchunks;         // activation rows are handled in chunks
-    int n_blocks;        // workgroups of this problem in the flat grid
     // Look-up kernel: the (tile, set) items of one row chunk, tile-major, are cut
     // into `wgs_per_chunk` contiguous ranges of `items_per_wg` items.
     int items_per_wg;
     int wgs_per_chunk;
+    int mchunks;         // activation rows are handled in chunks
+    int n_blocks;        // workgroups of this problem
     // Matrix-core kernel: K-steps per K-slice and slices per tile.
     int sets_per_split;
     int ksplit;
-    int finish;          // kFinishInline / kFinishDefer
-    // fused input transforms and output mode (row-wise look-up path only)
-    const __half *norm_w;  // non-null: the input is fp16(fp16(x * rsqrt(mean(x^2) + norm_eps)) * norm_w)
-    const __half *gate;    // non-null [M][K]: the input is fp16(fp16(silu(gate)) * x)
+    int sumsq_slots;
+    int R;               // block modes: row groups
+    int rows_per_group;  // block modes: N / R
     float norm_eps;
-    int overwrite;         // 1: out = y instead of out += y
+    // fused input transforms (row-wise look-up path only)
+    const __half *norm_w;  // non-null: y = rsqrt(mean(x^2) + norm_eps) * W(fp16(x * norm_w))
+    const __half *gate;    // non-null [M][K]: the input is fp16(fp16(silu(gate)) * x)
+    const __half *qbias;
+    // ---- needed when sums are handed over ------------------------------------------------
+    __half *out;
+    unsigned long long *accum;  // [M][N] fixed-point words, zero between launches
+    int finish;          // kFinishInline / kFinishDefer
+    int overwrite;       // 1: out = y instead of out += y
+    // RMSNorm split over two launches (fused entry point only).  The launch that completes
+    // a residual row also leaves next_in = fp16(out * next_w) and adds the squares of its
+    // outputs, 32 columns at a time, into sumsq_out[m][n / 32]; the launch that consumes
+    // next_in scales its sums by rsqrt(sum(sumsq_in[m][0 .. sumsq_slots)) / K + norm_eps).
+    const __half *next_w;   // [N]
+    __half *next_in;        // [M][N]
+    float *sumsq_out;       // [M][N / 32], zero before the launch
 };
 
 struct Group {
@@ -152,6 +166,29 @@ __device__ __forceinline__ float half_bits_to_float(uint32_t bits16)
 __device__ __forceinline__ uint32_t float_to_half_bits(float f)
 {
     return (uint32_t)__half_as_ushort(__float2half_rn(f));
+}
+
+// The value of another lane of the same row of 16, by a data-parallel-primitive move.
+template <int CTRL>
+__device__ __forceinline__ float dpp_move(float v)
+{
+    const int vi = __builtin_bit_cast(int, v);
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(vi, vi, CTRL, 0xf, 0xf, false));
+}
+
+// Sum over the 64 lanes of a wave, on the vector ALU: xor 1 and 2 inside quads, then the
+// mirrored quad and the mirrored half of each row of 16, then the four rows.
+__device__ __forceinline__ float wave_sum(float v)
+{
+    v += dpp_move<0xb1>(v);   // quad_perm [1,0,3,2]
+    v += dpp_move<0x4e>(v);   // quad_perm [2,3,0,1]
+    v += dpp_move<0x141>(v);  // row_half_mirror
+    v += dpp_move<0x140>(v);  // row_mirror
+    const int vi = __builtin_bit_cast(int, v);
+    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(vi, 0)) +
+           __builtin_bit_cast(float, __builtin_amdgcn_readlane(vi, 16)) +
+           __builtin_bit_cast(float, __builtin_amdgcn_readlane(vi, 32)) +
+           __builtin_bit_cast(float, __builtin_amdgcn_readlane(vi, 48));
 }
 
 // One partial sum as a contribution to an accumulator word: the addend, and the

@@ -293,8 +293,7 @@ int run_mfma_group(Group &g, const Accum &acc)
         Problem &p = g.p[i];
         const long mine = (long)p.N * (p.K / 8) * p.nb;
         plan_mfma(p, mt, (long)mfma_blocks(mt) * mine / (total_bytes > 0 ? total_bytes : 1));
-        p.block_begin = begin;
-        begin += p.n_blocks;
+        if (p.n_blocks > begin) begin = p.n_blocks;  // grid.x: the largest problem's workgroups
         any_split = any_split || p.ksplit > 1;
     }
     if (any_split) {
@@ -307,7 +306,7 @@ int run_mfma_group(Group &g, const Accum &acc)
             off += (size_t)g.p[i].M * g.p[i].N;
         }
     }
-    const hipError_t e = launch_mfma_group(g, mt, begin, acc.stream);
+    const hipError_t e = g.count == 1 ? launch_mfma_fused(g.p[0], mt, acc.stream) : launch_mfma_group(g, mt, begin, acc.stream);
     return e == hipSuccess ? LUTGEMM_OK : hip_fail(e);
 }
 
@@ -360,11 +359,24 @@ int run_group(int count, const lutgemm_fused_problem *problems, const Accum &acc
         p.gate = (const __half *)q.gate_f16;
         p.norm_eps = q.norm_eps;
         p.overwrite = q.overwrite;
+        // RMSNorm split over two launches
+        if ((q.next_input_f16 != nullptr) != (q.next_norm_weight_f16 != nullptr)) return LUTGEMM_EINVAL;
+        if (q.sumsq_out_f32 && q.N % 32 != 0) return LUTGEMM_EINVAL;
+        if (q.sumsq_in_f32 && (q.sumsq_in_slots <= 0 || q.norm_weight_f16 || !(q.norm_eps >= 0.0f))) return LUTGEMM_EINVAL;
+        if (!q.sumsq_in_f32 && q.sumsq_in_slots != 0) return LUTGEMM_EINVAL;
+        if (!aligned(q.next_input_f16, 2) || !aligned(q.next_norm_weight_f16, 2) || !aligned(q.sumsq_out_f32, 4) ||
+            !aligned(q.sumsq_in_f32, 16))
+            return LUTGEMM_EALIGN;
+        p.next_w = (const __half *)q.next_norm_weight_f16;
+        p.next_in = (__half *)q.next_input_f16;
+        p.sumsq_out = q.sumsq_out_f32;
+        p.sumsq_in = q.sumsq_in_f32;
+        p.sumsq_slots = q.sumsq_in_slots;
         // one kernel instance per transform: the problems of a launch share theirs
         const int mine = p.norm_w ? kXNorm : p.gate ? kXGate : kXNone;
         if (i > 0 && mine != xform) return LUTGEMM_EUNSUP;
         xform = mine;
-        plain = plain && !p.norm_w && !p.gate && !p.overwrite;
+        plain = plain && !p.norm_w && !p.gate && !p.overwrite && !p.next_in && !p.sumsq_out && !p.sumsq_in;
         all_mfma = all_mfma && mfma_eligible(p, kRowF16);
         words += (size_t)q.M * q.N;
         total_bytes += (long)q.N * (q.K / 8) * q.nb * q.M;
@@ -402,8 +414,7 @@ int run_group(int count, const lutgemm_fused_problem *problems, const Accum &acc
         if (want < 1) want = 1;
         int rc = plan_lookup(p, 1, want);
         if (rc != LUTGEMM_OK) return rc;
-        p.block_begin = begin;
-        begin += p.n_blocks;
+        if (p.n_blocks > begin) begin = p.n_blocks;  // grid.x: the largest problem's workgroups
         any_split = any_split || lookup_splits_k(p);
     }
     if (any_split) {
@@ -416,7 +427,7 @@ int run_group(int count, const lutgemm_fused_problem *problems, const Accum &acc
             off += (size_t)g.p[i].M * g.p[i].N;
         }
     }
-    const hipError_t e = launch_gemv_group(g, xform, begin, acc.stream);
+    const hipError_t e = count == 1 ? launch_gemv_fused(g.p[0], xform, acc.stream) : launch_gemv_group(g, xform, begin, acc.stream);
     return e == hipSuccess ? LUTGEMM_OK : hip_fail(e);
 }
 

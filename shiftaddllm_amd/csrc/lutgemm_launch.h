@@ -11,10 +11,14 @@ namespace lutgemm {
 hipError_t launch_gemv_rowwise(const Problem &p, int mode, int mrows, hipStream_t stream);       // kRowF16, kUniformF16
 hipError_t launch_gemv_block(const Problem &p, int mode, int mrows, hipStream_t stream);         // kBlock*
 hipError_t launch_gemv_block_staged(const Problem &p, int mode, int mrows, hipStream_t stream);  // kBlock*Staged
-// look-up kernel, several row-wise problems, flat grid of `blocks` workgroups
+// look-up kernel, one row-wise problem with fused extras, one row per workgroup;
+// grid = (p.wgs_per_chunk, p.mchunks)
+hipError_t launch_gemv_fused(const Problem &p, int xform, hipStream_t stream);
+// look-up kernel, several row-wise problems; grid = (blocks of the largest problem, problems)
 hipError_t launch_gemv_group(const Group &g, int xform, int blocks, hipStream_t stream);
 // matrix-core kernel; mt = 1 (16-row tiles) or 2 (32-row tiles)
 hipError_t launch_mfma(const Problem &p, int mt, hipStream_t stream);
+hipError_t launch_mfma_fused(const Problem &p, int mt, hipStream_t stream);  // one problem with fused extras
 hipError_t launch_mfma_group(const Group &g, int mt, int blocks, hipStream_t stream);
 
 }  // namespace lutgemm

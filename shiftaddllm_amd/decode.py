@@ -103,9 +103,13 @@ class LutDecoder(nn.Module):
         if glue not in ("hip", "torch"):
             raise ValueError(f"glue must be 'hip' or 'torch', got {glue!r}")
         self.cfg, self.batch, self.fuse, self.glue = cfg, batch, fuse_launches, glue
-        # RMSNorm inside the q,k,v and gate,up GEMVs instead of a kernel of its own: measured equal
-        # (every workgroup re-reads the row to form its RMS), so the separate kernel stays the default
+        # RMSNorm inside the q,k,v and gate,up GEMVs instead of a kernel of its own (every workgroup
+        # re-reads the row to form its RMS: measured no faster than the separate kernel)
         self.fold_norm = False
+        # RMSNorm split over the GEMV that completes the residual row (it leaves x * norm weight and
+        # the row's sums of squares) and the GEMVs that read it (they scale their sums): no norm
+        # launches inside the stack, for any batch size
+        self.split_norm = fuse_launches and cfg.hidden % 32 == 0
         dev = torch.device(device)
         gen = torch.Generator(device=dev).manual_seed(seed)
         names = ("self_attn.q_proj", "self_attn.k_proj", "self_attn.v_proj", "self_attn.o_proj",
@@ -142,6 +146,8 @@ class LutDecoder(nn.Module):
         self.register_buffer("att", torch.zeros((batch, H), **f16), persistent=False)
         self.register_buffer("gate_up", torch.zeros((2 * batch * I,), **f16), persistent=False)
         self.register_buffer("act", torch.zeros((batch, I), **f16), persistent=False)
+        self.register_buffer("sumsq", torch.zeros((2 * cfg.layers, batch, max(cfg.hidden // 32, 1)),
+                                                  dtype=torch.float32, device=dev), persistent=False)
         self._graph = None
         self._stream = None
 
@@ -195,16 +201,20 @@ class LutDecoder(nn.Module):
             if rc:
                 raise RuntimeError(lib.lutgemm_strerror(rc).decode())
 
-    def _fused_gemv(self, lins, x, outs, sp, norm=None, gate=None, overwrite=False):
+    def _fused_gemv(self, lins, x, outs, sp, norm=None, gate=None, overwrite=False, next_norm=None, next_in=None,
+                    sumsq_out=None, sumsq_in=None):
         """One launch: outs[i] (+)= lins[i](t(x)), t = RMSNorm with weight `norm`, or
-        silu(gate) * x, or identity."""
+        silu(gate) * x, or identity.  next_norm / next_in / sumsq_out: the outputs complete
+        a residual row whose norm-weighted copy and sums of squares are left for the next
+        GEMV; sumsq_in: x is such a copy and the sums are scaled by its reciprocal RMS."""
         lib, B = native.cabi(), x.shape[0]
+        ptr = lambda t: t.data_ptr() if t is not None else None
         arr = (native.FusedProblem * len(lins))()
         for i, (l, o) in enumerate(zip(lins, outs)):
             arr[i] = native.FusedProblem(l.binaryWeight.data_ptr(), l.alpha.data_ptr(), x.data_ptr(), o.data_ptr(),
-                                         l.N, l.K, l.wbit, l.num_groups, B, int(overwrite),
-                                         norm.data_ptr() if norm is not None else None,
-                                         gate.data_ptr() if gate is not None else None, self.cfg.rms_eps)
+                                         l.N, l.K, l.wbit, l.num_groups, B, int(overwrite), ptr(norm), ptr(gate),
+                                         self.cfg.rms_eps, ptr(next_norm), ptr(next_in), ptr(sumsq_out),
+                                         ptr(sumsq_in), sumsq_in.shape[-1] if sumsq_in is not None else 0)
         rc = lib.lutgemm_gemv_rowwise_f16_fused(len(lins), arr, sp)
         if rc:
             raise RuntimeError(lib.lutgemm_strerror(rc).decode())
@@ -230,46 +240,56 @@ class LutDecoder(nn.Module):
         fold = self.fuse
         fold_gate = fold and B <= 2                         # input transforms live in the look-up kernel
         fold_norm = fold_gate and self.fold_norm
+        split = fold and self.split_norm and not fold_norm
+        rmsnorm = lambda w, clear=None: check(lib.lutgemm_decode_rmsnorm_f16(
+            x.data_ptr(), w.data_ptr(), h.data_ptr(), B, cfg.hidden, cfg.rms_eps,
+            clear.data_ptr() if clear is not None else None, clear.numel() * 2 if clear is not None else 0, sp))
         torch.index_select(self.embed, 0, self.ids, out=x)
+        if split:
+            self.sumsq.zero_()
         for li, blk in enumerate(self.blocks):
             qkv_lins = [blk.q_proj, blk.k_proj, blk.v_proj]
-            if fold_norm:
+            if split and li > 0:                                        # h, sums: left by the last down_proj
+                self._fused_gemv(qkv_lins, h, [q, k, v], sp, overwrite=True, sumsq_in=self.sumsq[2 * li - 1])
+            elif fold_norm:
                 self._fused_gemv(qkv_lins, x, [q, k, v], sp, norm=blk.input_norm, overwrite=True)
             elif fold:
-                check(lib.lutgemm_decode_rmsnorm_f16(x.data_ptr(), blk.input_norm.data_ptr(), h.data_ptr(), B,
-                                                     cfg.hidden, cfg.rms_eps, None, 0, sp))
+                rmsnorm(blk.input_norm)
                 self._fused_gemv(qkv_lins, h, [q, k, v], sp, overwrite=True)
             else:
-                check(lib.lutgemm_decode_rmsnorm_f16(x.data_ptr(), blk.input_norm.data_ptr(), h.data_ptr(), B,
-                                                     cfg.hidden, cfg.rms_eps, self.qkv.data_ptr(),
-                                                     self.qkv.numel() * 2, sp))
+                rmsnorm(blk.input_norm, self.qkv)
                 self._gemv_into(qkv_lins, h, [q, k, v], sp)
             check(lib.lutgemm_decode_attention_f16(q.data_ptr(), k.data_ptr(), v.data_ptr(), self.cos.data_ptr(),
                                                    self.sin.data_ptr(), self.k_cache[li].data_ptr(),
                                                    self.v_cache[li].data_ptr(), self.pos.data_ptr(),
                                                    self.att.data_ptr(), B, H, KV, hd, cfg.max_positions, sp))
-            self._gemv_into([blk.o_proj], self.att, [x], sp)            # x += o_proj(att)
-            if fold:
-                if fold_norm:
-                    self._fused_gemv([blk.gate_proj, blk.up_proj], x, [g, u], sp, norm=blk.post_norm, overwrite=True)
-                else:
-                    check(lib.lutgemm_decode_rmsnorm_f16(x.data_ptr(), blk.post_norm.data_ptr(), h.data_ptr(), B,
-                                                         cfg.hidden, cfg.rms_eps, None, 0, sp))
-                    self._fused_gemv([blk.gate_proj, blk.up_proj], h, [g, u], sp, overwrite=True)
-                if fold_gate:
-                    self._fused_gemv([blk.down_proj], u, [x], sp, gate=g)   # x += down_proj(silu(g) * u)
-                else:
-                    check(lib.lutgemm_decode_silu_mul_f16(g.data_ptr(), u.data_ptr(), self.act.data_ptr(), B * I, sp))
-                    self._gemv_into([blk.down_proj], self.act, [x], sp)
+            gate_up = [blk.gate_proj, blk.up_proj]
+            if split:                                                   # x += o_proj(att); h = x * post_norm
+                self._fused_gemv([blk.o_proj], self.att, [x], sp, next_norm=blk.post_norm, next_in=h,
+                                 sumsq_out=self.sumsq[2 * li])
+                self._fused_gemv(gate_up, h, [g, u], sp, overwrite=True, sumsq_in=self.sumsq[2 * li])
             else:
-                check(lib.lutgemm_decode_rmsnorm_f16(x.data_ptr(), blk.post_norm.data_ptr(), h.data_ptr(), B,
-                                                     cfg.hidden, cfg.rms_eps, self.gate_up.data_ptr(),
-                                                     self.gate_up.numel() * 2, sp))
-                self._gemv_into([blk.gate_proj, blk.up_proj], h, [g, u], sp)
+                self._gemv_into([blk.o_proj], self.att, [x], sp)        # x += o_proj(att)
+                if fold_norm:
+                    self._fused_gemv(gate_up, x, [g, u], sp, norm=blk.post_norm, overwrite=True)
+                elif fold:
+                    rmsnorm(blk.post_norm)
+                    self._fused_gemv(gate_up, h, [g, u], sp, overwrite=True)
+                else:
+                    rmsnorm(blk.post_norm, self.gate_up)
+                    self._gemv_into(gate_up, h, [g, u], sp)
+            # x += down_proj(silu(g) * u), leaving the next block's normalised input behind
+            nxt = dict(next_norm=self.blocks[li + 1].input_norm, next_in=h, sumsq_out=self.sumsq[2 * li + 1]) \
+                if split and li + 1 < len(self.blocks) else {}
+            if fold_gate:
+                self._fused_gemv([blk.down_proj], u, [x], sp, gate=g, **nxt)
+            else:
                 check(lib.lutgemm_decode_silu_mul_f16(g.data_ptr(), u.data_ptr(), self.act.data_ptr(), B * I, sp))
-                self._gemv_into([blk.down_proj], self.act, [x], sp)     # x += down_proj(act)
-        check(lib.lutgemm_decode_rmsnorm_f16(x.data_ptr(), self.final_norm.data_ptr(), h.data_ptr(), B, cfg.hidden,
-                                             cfg.rms_eps, None, 0, sp))
+                if nxt:
+                    self._fused_gemv([blk.down_proj], self.act, [x], sp, **nxt)
+                else:
+                    self._gemv_into([blk.down_proj], self.act, [x], sp)
+        rmsnorm(self.final_norm)
         torch.matmul(h, self.lm_head.t(), out=self.logits)
 
     def _step_torch(self):

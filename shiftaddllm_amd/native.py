@@ -58,7 +58,10 @@ class FusedProblem(ctypes.Structure):
                 ("out_f16", ctypes.c_void_p), ("N", ctypes.c_int), ("K", ctypes.c_int),
                 ("nb", ctypes.c_int), ("num_groups", ctypes.c_int), ("M", ctypes.c_int),
                 ("overwrite", ctypes.c_int), ("norm_weight_f16", ctypes.c_void_p),
-                ("gate_f16", ctypes.c_void_p), ("norm_eps", ctypes.c_float)]
+                ("gate_f16", ctypes.c_void_p), ("norm_eps", ctypes.c_float),
+                ("next_norm_weight_f16", ctypes.c_void_p), ("next_input_f16", ctypes.c_void_p),
+                ("sumsq_out_f32", ctypes.c_void_p), ("sumsq_in_f32", ctypes.c_void_p),
+                ("sumsq_in_slots", ctypes.c_int)]
 
 
 class NativeLibraryMissing(ImportError):

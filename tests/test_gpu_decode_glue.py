@@ -223,3 +223,79 @@ def test_overwrite_mode_ignores_previous_output(gpu_device, M):
     torch.cuda.synchronize()
     for a, b in zip(got, want):
         assert torch.allclose(a.float(), b.float(), rtol=2e-3, atol=2e-3 * float(b.float().abs().max()))
+
+
+# ---- RMSNorm split over the completing and the consuming GEMV ---------------------------
+
+def _split_call(lib, lin, x, out, M, **kw):
+    bW, alpha, N, K, nb = lin
+    ptr = lambda t: t.data_ptr() if t is not None else None
+    arr = (native.FusedProblem * 1)()
+    arr[0] = native.FusedProblem(bW.data_ptr(), alpha.data_ptr(), x.data_ptr(), out.data_ptr(), N, K, nb, K // 128, M,
+                                 int(kw.get("overwrite", False)), None, ptr(kw.get("gate")), 1e-5,
+                                 ptr(kw.get("next_norm")), ptr(kw.get("next_in")), ptr(kw.get("sumsq_out")),
+                                 ptr(kw.get("sumsq_in")), kw["sumsq_in"].shape[-1] if kw.get("sumsq_in") is not None else 0)
+    return lib.lutgemm_gemv_rowwise_f16_fused(1, arr, _sp())
+
+
+@pytest.mark.parametrize("M", [1, 2, 8, 20])                 # look-up kernel (1, 2 rows), matrix cores (16- and 32-row tiles)
+@pytest.mark.parametrize("N,K,N2,nb", [(1024, 2048, 768, 3), (4096, 1408 - 1408 % 128, 512, 4)])
+def test_split_rmsnorm_equals_separate_kernels(gpu_device, M, N, K, N2, nb):
+    """GEMV 1 completes a residual row and leaves (row * weight, sums of squares); GEMV 2
+    reads those: together they equal GEMV, rmsnorm kernel, GEMV."""
+    lib = native.cabi()
+    g = torch.Generator(device=gpu_device).manual_seed(M * 31 + N)
+    a = torch.randn((M, K), generator=g, device=gpu_device).half()
+    res = (torch.randn((M, N), generator=g, device=gpu_device) * 3).half()
+    w = (1 + 0.2 * torch.randn((N,), generator=g, device=gpu_device)).half()
+    lin1, lin2 = _random_lin(gpu_device, N, K, nb, 3), _random_lin(gpu_device, N2, N, 3, 4)
+
+    # separate kernels
+    x_ref = res.clone()
+    _plain(lib, lin1, a, x_ref)
+    h_ref = torch.empty_like(x_ref)
+    _ok(lib.lutgemm_decode_rmsnorm_f16(x_ref.data_ptr(), w.data_ptr(), h_ref.data_ptr(), M, N, 1e-5, None, 0, _sp()))
+    y_ref = torch.zeros((M, N2), dtype=torch.float16, device=gpu_device)
+    _plain(lib, lin2, h_ref, y_ref)
+
+    # split norm
+    x = res.clone()
+    nxt = torch.full((M, N), 7.0, dtype=torch.float16, device=gpu_device)
+    sumsq = torch.zeros((M, N // 32), dtype=torch.float32, device=gpu_device)
+    _ok(_split_call(lib, lin1, a, x, M, next_norm=w, next_in=nxt, sumsq_out=sumsq))
+    y = torch.full((M, N2), 9.0, dtype=torch.float16, device=gpu_device)
+    _ok(_split_call(lib, lin2, nxt, y, M, overwrite=True, sumsq_in=sumsq))
+    torch.cuda.synchronize()
+
+    assert torch.allclose(x.float(), x_ref.float(), rtol=2e-3, atol=2e-3 * float(x_ref.float().abs().max()))
+    assert torch.equal(nxt, (x.float() * w.float()).half())                    # one rounding of an exact product
+    want_sq = x.float().pow(2).sum(-1)
+    assert torch.allclose(sumsq.sum(-1), want_sq, rtol=1e-5)
+    assert torch.allclose(y.float(), y_ref.float(), rtol=4e-3, atol=4e-3 * float(y_ref.float().abs().max()))
+
+
+def test_split_rmsnorm_with_swiglu_input_and_bad_arguments(gpu_device):
+    lib = native.cabi()
+    g = torch.Generator(device=gpu_device).manual_seed(77)
+    M, N, K = 1, 512, 1408 - 1408 % 128
+    gate = torch.randn((M, K), generator=g, device=gpu_device).half()
+    up = torch.randn((M, K), generator=g, device=gpu_device).half()
+    res = torch.randn((M, N), generator=g, device=gpu_device).half()
+    w = (1 + 0.2 * torch.randn((N,), generator=g, device=gpu_device)).half()
+    lin = _random_lin(gpu_device, N, K, 2, 9)
+    want = res.clone()
+    _ok(_fused_call(lib, [lin], up, [want], gate=gate))
+    x, nxt = res.clone(), torch.empty((M, N), dtype=torch.float16, device=gpu_device)
+    sumsq = torch.zeros((M, N // 32), dtype=torch.float32, device=gpu_device)
+    _ok(_split_call(lib, lin, up, x, M, gate=gate, next_norm=w, next_in=nxt, sumsq_out=sumsq))
+    torch.cuda.synchronize()
+    assert torch.equal(x, want)
+    assert torch.equal(nxt, (x.float() * w.float()).half())
+    assert torch.allclose(sumsq.sum(-1), x.float().pow(2).sum(-1), rtol=1e-5)
+    # the weight and the destination of the weighted copy come together
+    assert _split_call(lib, lin, up, x, M, next_in=nxt) == -1
+    assert _split_call(lib, lin, up, x, M, next_norm=w) == -1
+    # slots of 32 columns
+    lin_odd = _random_lin(gpu_device, 528, K, 2, 9)
+    x_odd = torch.zeros((M, 528), dtype=torch.float16, device=gpu_device)
+    assert _split_call(lib, lin_odd, up, x_odd, M, sumsq_out=sumsq) == -1
