@@ -422,8 +422,9 @@ __device__ __forceinline__ void gemv_range(const Problem &p, int range, int mchu
 
     // this workgroup's items; (tile, set) is the current one
     const int total = p.n_tiles * p.nsets;
-    const int item0 = range * p.items_per_wg;
-    int rem = min(p.items_per_wg, total - item0);
+    const bool long_range = range < p.long_ranges;
+    const int item0 = long_range ? range * p.items_per_wg : p.split_item + (range - p.long_ranges) * p.short_items;
+    int rem = min(long_range ? p.items_per_wg : p.short_items, total - item0);
     int tile = fast_div(item0, p.by_nsets), set = item0 - tile * p.nsets;
     auto advance = [&](int &t, int &s) {
         if (++s == p.nsets) {
@@ -557,9 +558,12 @@ __device__ __forceinline__ void gemv_range(const Problem &p, int range, int mchu
     // ---- hand a tile's complete K-slice over ---------------------------------------
     auto flush_tile = [&](int t) {
         // contributions this tile receives: the ranges that overlap its items
-        const int first = fast_div(t * p.nsets, p.by_items);
-        const int last = fast_div(t * p.nsets + p.nsets - 1, p.by_items);
-        const int count = last - first + 1;
+        auto range_of = [&](int item) {
+            const int in_long = fast_div(item, p.by_items);
+            const int in_short = p.long_ranges + fast_div(max(item - p.split_item, 0), p.by_short_items);
+            return item < p.split_item ? in_long : in_short;
+        };
+        const int count = range_of(t * p.nsets + p.nsets - 1) - range_of(t * p.nsets) + 1;
         int kw2 = kw;
         asm volatile("" : "+v"(kw2));  // (opaque: see own_col_of)
         const int n = t * kTileCols + own_col_of(kw2);

@@ -123,9 +123,14 @@ struct Problem {
     Divisor by_nsets;        // item / nsets
     Divisor by_items;        // item / items_per_wg
     // Look-up kernel: the (tile, set) items of one row chunk, tile-major, are cut
-    // into `wgs_per_chunk` contiguous ranges of `items_per_wg` items.
+    // into `wgs_per_chunk` contiguous ranges: the first `long_ranges` of `items_per_wg`
+    // items, the others, from item `split_item` on, of `short_items`.
     int items_per_wg;
     int wgs_per_chunk;
+    int long_ranges;
+    int short_items;
+    int split_item;          // long_ranges * items_per_wg
+    Divisor by_short_items;  // item / short_items
     int mchunks;         // activation rows are handled in chunks
     int n_blocks;        // workgroups of this problem
     // Matrix-core kernel: K-steps per K-slice and slices per tile.

@@ -145,8 +145,21 @@ int target_blocks(long sign_bytes)
     return sign_bytes <= (24l << 20) ? 256 : 512;  // 1 or 2 workgroups x 256 CUs
 }
 
-// Cut the (tile, set) items of a problem into equal contiguous ranges, one per
-// workgroup, aiming at `want_blocks` workgroups.
+// Of the two workgroups that share a CU the one dispatched first runs faster (the older
+// waves win the arbitration for issue slots and memory requests): with equal ranges the
+// first half of a 512-workgroup grid ends 6-7 us before the second on the 132 MB shapes.
+// So the first 256 workgroups get this share (per cent) of each pair's items.  Measured,
+// equal ranges vs 60 %: 28672x8192x2 17.3 vs 16.3 us, 8192x28672x2 17.1 vs 15.8, 8192x28672x4
+// 27.7 vs 27.0, 13824x5120x4 14.8 vs 13.1 (there mostly because 412 workgroups of 3 and 2
+// items fill the CUs better than 360 of 3), 8192x8192x4 unchanged.
+int first_share()
+{
+    static const int v = env_int("LUTGEMM_FIRST_SHARE", 60);
+    return v;
+}
+
+// Cut the (tile, set) items of a problem into contiguous ranges, one per workgroup,
+// aiming at `want_blocks` workgroups.
 int plan_lookup(Problem &p, int mrows, long want_blocks)
 {
     p.n_tiles = (p.N + kTileCols - 1) / kTileCols;
@@ -160,10 +173,29 @@ int plan_lookup(Problem &p, int mrows, long want_blocks)
     const long cap = (p.nsets + kMaxContrib - 2) / (kMaxContrib - 1);
     if (ipw < cap) ipw = cap;
     if (ipw > total) ipw = total;
+    long n_long = (total + ipw - 1) / ipw, short_items = ipw, n_short = 0;
+    // two resident workgroups per CU, one row chunk: unequal shares within each pair
+    const int share = first_share();
+    if (p.mchunks == 1 && want_blocks == 512 && total >= 2 * 256 * 2 && share > 50 && share < 100) {
+        const long pair = (total + 255) / 256;
+        long a = (pair * share + 99) / 100, b = pair - a;
+        if (b >= 1 && b >= cap && a > b) {
+            ipw = a;
+            n_long = 256;
+            short_items = b;
+            const long rest = total - n_long * a;
+            n_short = rest > 0 ? (rest + b - 1) / b : 0;
+            if (rest <= 0) n_long = (total + a - 1) / a;
+        }
+    }
     p.items_per_wg = (int)ipw;
-    p.wgs_per_chunk = (int)((total + ipw - 1) / ipw);
+    p.long_ranges = (int)n_long;
+    p.short_items = (int)short_items;
+    p.split_item = (int)(n_long * ipw);
+    p.wgs_per_chunk = (int)(n_long + n_short);
     p.n_blocks = p.wgs_per_chunk * p.mchunks;
     p.by_items = make_divisor(p.items_per_wg);
+    p.by_short_items = make_divisor(p.short_items);
     p.by_nsets = make_divisor(p.nsets);
     // the multiply-high divisions of the kernel are exact within this bound
     if (2ull * (unsigned long long)(total + p.nsets) * (unsigned long long)ipw >= (1ull << 32)) return LUTGEMM_EUNSUP;
@@ -171,7 +203,11 @@ int plan_lookup(Problem &p, int mrows, long want_blocks)
 }
 
 // true when some tile is shared between ranges, i.e. accumulator words are needed
-bool lookup_splits_k(const Problem &p) { return p.items_per_wg % p.nsets != 0 || p.finish == kFinishDefer; }
+bool lookup_splits_k(const Problem &p)
+{
+    if (p.finish == kFinishDefer || p.items_per_wg % p.nsets != 0) return true;
+    return p.wgs_per_chunk > p.long_ranges && (p.short_items % p.nsets != 0 || p.split_item % p.nsets != 0);
+}
 
 int pick_mrows(int M) { return M >= 3 ? 4 : M; }
 
