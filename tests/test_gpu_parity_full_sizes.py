@@ -77,6 +77,17 @@ def test_config5_small_batches_full_size(gpu_device, N, K, nb, M):
     _assert_close(run_rowwise(gpu_device, bW, alpha, x), want, (N, K, nb, M))
 
 
+@pytest.mark.parametrize("N,K,nb,group", [(9000, 8224, 4, 32), (13824, 5120, 4, 128), (25604, 4128, 3, 32)])
+def test_ragged_shapes_on_unequal_ranges(gpu_device, N, K, nb, group):
+    """More than 24 MB of signs: 512 workgroups whose ranges come in two sizes (the
+    workgroup dispatched first on a CU takes the larger share), here with a last tile
+    and a last set that are only partly filled."""
+    print(f"ragged N={N} K={K} nb={nb}", flush=True)
+    bW, alpha, x = packed_rowwise(N, K, nb, 1, seed=N + K, group=group)
+    want, _ = orc.gemv_rowwise_c(bW.numpy(), alpha.numpy(), x.numpy(), K // group)
+    _assert_close(run_rowwise(gpu_device, bW, alpha, x, group=group), want, (N, K, nb))
+
+
 # ---- config 3: Llama-2-13B shapes in the integer alpha formats -----------------------
 
 @pytest.mark.parametrize("kind", ["apot_i8", "shift_u16"])
