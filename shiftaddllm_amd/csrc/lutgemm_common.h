@@ -5,6 +5,7 @@
 
 #include <hip/hip_runtime.h>
 #include <hip/hip_fp16.h>
+#include <stddef.h>
 #include <stdint.h>
 
 #include "lutgemm_gfx950.h"
@@ -108,7 +109,7 @@ __device__ __forceinline__ int fast_div(int n, const Divisor &d)
 // trip on the start-up path.  What the kernels need to issue their first loads comes
 // first (two 64-byte lines), what the hand-over of finished sums needs comes last.
 struct Problem {
-    // ---- needed to request the first operands -----------------------------------------
+    // ---- cache line 0: every kernel's first requests ---------------------------------------
     const uint32_t *W;
     const void *alpha;
     const __half *x;
@@ -119,35 +120,36 @@ struct Problem {
     int n_tiles;
     int group_words;     // row-wise / uniform: words per alpha group
     int nb;
+    // ---- cache line 1: the rest of what is needed to request the first operands ------------
     Divisor by_group_words;  // row / group_words
     Divisor by_nsets;        // item / nsets
-    Divisor by_items;        // item / items_per_wg
     // Look-up kernel: the (tile, set) items of one row chunk, tile-major, are cut
     // into `wgs_per_chunk` contiguous ranges: the first `long_ranges` of `items_per_wg`
     // items, the others, from item `split_item` on, of `short_items`.
     int items_per_wg;
-    int wgs_per_chunk;
     int long_ranges;
     int short_items;
-    int split_item;          // long_ranges * items_per_wg
-    Divisor by_short_items;  // item / short_items
+    int split_item;      // long_ranges * items_per_wg
     int mchunks;         // activation rows are handled in chunks
     int n_blocks;        // workgroups of this problem
-    // Matrix-core kernel: K-steps per K-slice and slices per tile.
-    int sets_per_split;
-    int ksplit;
+    int wgs_per_chunk;
     int sumsq_slots;
     int R;               // block modes: row groups
     int rows_per_group;  // block modes: N / R
-    float norm_eps;
-    // fused input transforms (row-wise look-up path only)
     const __half *norm_w;  // non-null: y = rsqrt(mean(x^2) + norm_eps) * W(fp16(x * norm_w))
+    // ---- cache line 2 ----------------------------------------------------------------------
     const __half *gate;    // non-null [M][K]: the input is fp16(fp16(silu(gate)) * x)
     const __half *qbias;
-    // ---- needed when sums are handed over ------------------------------------------------
     __half *out;
     unsigned long long *accum;  // [M][N] fixed-point words, zero between launches
+    Divisor by_items;        // item / items_per_wg
+    Divisor by_short_items;  // item / short_items
+    // Matrix-core kernel: K-steps per K-slice and slices per tile.
+    int sets_per_split;
+    int ksplit;
+    float norm_eps;
     int finish;          // kFinishInline / kFinishDefer
+    // ---- cache line 3: needed when sums are handed over --------------------------------------
     int overwrite;       // 1: out = y instead of out += y
     // RMSNorm split over two launches (fused entry point only).  The launch that completes
     // a residual row also leaves next_in = fp16(out * next_w) and adds the squares of its
@@ -157,6 +159,8 @@ struct Problem {
     __half *next_in;        // [M][N]
     float *sumsq_out;       // [M][N / 32], zero before the launch
 };
+static_assert(offsetof(Problem, by_group_words) == 64 && offsetof(Problem, gate) == 128 && offsetof(Problem, overwrite) == 192,
+              "Problem: fields are grouped by cache line");
 
 struct Group {
     int count;
