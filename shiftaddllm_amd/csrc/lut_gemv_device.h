@@ -422,9 +422,10 @@ __device__ __forceinline__ void gemv_range(const Problem &p, int range, int mchu
 
     // this workgroup's items; (tile, set) is the current one
     const int total = p.n_tiles * p.nsets;
-    const bool long_range = range < p.long_ranges;
-    const int item0 = long_range ? range * p.items_per_wg : p.split_item + (range - p.long_ranges) * p.short_items;
-    int rem = min(long_range ? p.items_per_wg : p.short_items, total - item0);
+    // (branch-free: a branch here becomes one more round of scalar loads ahead of the first requests)
+    const int beyond = range - p.long_ranges;  // >= 0: a short range
+    const int item0 = min(range, p.long_ranges) * p.items_per_wg + max(beyond, 0) * p.short_items;
+    int rem = min(p.short_items + (beyond < 0 ? p.items_per_wg - p.short_items : 0), total - item0);
     int tile = fast_div(item0, p.by_nsets), set = item0 - tile * p.nsets;
     auto advance = [&](int &t, int &s) {
         if (++s == p.nsets) {
