@@ -95,7 +95,8 @@ struct ItemOperands {
 // with every lane pointed at the first words of the operands: a handful of cache
 // lines instead of a conditional load.  Addresses are a uniform 64-bit base plus a
 // 32-bit per-lane offset.
-template <int NB, int MODE>
+// PARTS: 1 = the sign words only, 2 = everything else (alphas), 3 = both.
+template <int NB, int MODE, int PARTS = 3>
 __device__ __forceinline__ void load_item(ItemOperands<NB, MODE> &r, const Problem &p, int tile, int set, bool valid,
                                           int kw, int q, int lane_col, int tid)
 {
@@ -112,11 +113,14 @@ __device__ __forceinline__ void load_item(ItemOperands<NB, MODE> &r, const Probl
     [[maybe_unused]] const int row = set * kSetWords + kwc;
     [[maybe_unused]] const int g = fast_div(row, p.by_group_words);  // alpha group of the row
     const uint32_t woff = (wrow + col4) & lane_mask;
+    if constexpr (PARTS & 1) {
 #pragma unroll
-    for (int b = 0; b < NB; ++b) {
-        const char *src = wbase + (size_t)b * row_bytes;
-        r.w[b] = __builtin_nontemporal_load((const u32x4 *)(src + woff));
+        for (int b = 0; b < NB; ++b) {
+            const char *src = wbase + (size_t)b * row_bytes;
+            r.w[b] = __builtin_nontemporal_load((const u32x4 *)(src + woff));
+        }
     }
+    if constexpr (!(PARTS & 2)) return;
     if constexpr (MODE == kRowF16) {
         const uint32_t aoff = ((uint32_t)g * (NB * (uint32_t)p.N * 2u) + col2) & lane_mask;
 #pragma unroll
@@ -500,7 +504,6 @@ __device__ __forceinline__ void gemv_range(const Problem &p, int range, int mchu
             lane_off |= (uint32_t)(4 * (lkw * 4 + jj)) << (8 * j);
             sel[j] = 0x0c0c0000u | ((uint32_t)(4 + jj) << 8) | (uint32_t)j;
         }
-        fetch_out(tile);
     };
     // Also once, after that: park the first window and, with a fused RMSNorm, leave each
     // wave's share of the rows' sums of squares in LDS.  The reciprocal RMS is formed
@@ -639,7 +642,8 @@ __device__ __forceinline__ void gemv_range(const Problem &p, int range, int mchu
     constexpr uint32_t kFlip = 0x80808080u;  // +128 bytes = the other table buffer
     int buf = 0;
     int rel = 0;  // items of the range done so far
-    auto item_step = [&](const ItemOperands<NB, MODE> &ops, bool last) {
+    // `after_first_barrier` runs behind the barrier of the item's first row (see the first item below).
+    auto item_step = [&](const ItemOperands<NB, MODE> &ops, bool last, auto &&after_first_barrier) {
         int nt = tile, ns = set;
         advance(nt, ns);
         const int slot = rel % kSlots;
@@ -665,6 +669,11 @@ __device__ __forceinline__ void gemv_range(const Problem &p, int range, int mchu
             build_tables(xr, lut, buf, tb, eb);
             if (r == 0) stage_alpha<NB, MODE>(ops, stage, abuf, tid);
             __syncthreads();
+            if (r == 0) {
+                __builtin_amdgcn_sched_barrier(0);
+                after_first_barrier();
+                __builtin_amdgcn_sched_barrier(0);
+            }
             // opaque to the optimiser: otherwise the look-up addresses of an item are
             // kept in registers across all rows instead of being recomputed (1 op each)
             asm volatile("" : "+v"(lane_off));
@@ -682,37 +691,79 @@ __device__ __forceinline__ void gemv_range(const Problem &p, int range, int mchu
         set = ns;
     };
     // Two operand buffers alternate: while one item is processed the next one's loads
-    // are in flight, and the first two items of the range are requested before anything
-    // is waited for.  Items are taken in pairs by a counted loop with ONE exit and ONE
-    // load site per buffer:
-    //  * with a second load site (a prologue, say) the register allocator gives the two
-    //    sites different registers and reconciles them with copies that wait for the loads;
+    // are in flight.
+    //
+    // The FIRST item is taken outside the loop, and as little as possible is requested
+    // before its tables stand.  A CU keeps only so many vector memory instructions in
+    // flight (about 64, all waves together); a wave whose next load does not fit stalls at
+    // that instruction, whatever else it could do.  With everything requested up front
+    // (activations, two items, the caller's outputs: 15 loads per wave at three bit
+    // planes) the second wave of every SIMD got stuck behind the first one's loads and
+    // reached its table build a memory latency late (measured per wave: activations usable
+    // at 1.3 us in waves 0-3, at 2.1 us in waves 4-7, and the workgroup's first barrier
+    // waits for the last).  So: activations and the first item's sign words first; its
+    // alphas once the activation window is parked; the second item and the caller's
+    // outputs behind the first barrier.  4096x4096 3-bit: 5.98 -> 4.93 us per call.
+    //
+    // The other items are taken in pairs by a counted loop with ONE exit and one load site
+    // per buffer inside it:
+    //  * with a second load site in the loop the register allocator gives the two sites
+    //    different registers and reconciles them with copies that wait for the loads;
     //  * with a second exit the loop is restructured with edges that are never taken but
     //    on which loads are still pending, and every iteration then starts by waiting
     //    for everything in flight.
-    // Hence the first iteration skips its first step at run time, and the second item of
-    // the last pair, if the range has an odd number of items, is a dummy (see load_item).
+    // An item that does not exist (the second of the last pair of an odd range) is requested
+    // as a dummy (see load_item).
     ItemOperands<NB, MODE> opA, opB;
     int ld_tile = tile, ld_set = set;  // next item to request
     const int pairs = (n_items + 1) / 2;
+    auto no_hook = []() {};
+    if constexpr (MROWS == 1 && !is_block(MODE)) {
+        load_item<NB, MODE, 1>(opA, p, ld_tile, ld_set, true, kw, q, lane_col, tid);
+        __builtin_amdgcn_sched_barrier(0);
+        late_setup();
+        first_window();
+        load_item<NB, MODE, 2>(opA, p, ld_tile, ld_set, true, kw, q, lane_col, tid);
+        advance(ld_tile, ld_set);
+        item_step(opA, n_items == 1, [&]() {
+            fetch_out(tile);
+            load_item<NB, MODE>(opB, p, ld_tile, ld_set, 1 < n_items, kw, q, lane_col, tid);
+            advance(ld_tile, ld_set);
+        });
 #pragma clang loop unroll(disable)
-    for (int j = 0; j < pairs; ++j) {
-        // (opaque, which keeps the compiler from peeling the first iteration)
-        int first = __builtin_amdgcn_readfirstlane(j == 0);
-        asm volatile("" : "+s"(first));
-        load_item<NB, MODE>(opA, p, ld_tile, ld_set, true, kw, q, lane_col, tid);
-        advance(ld_tile, ld_set);
-        if (!first) item_step(opB, false);
-        const bool has_b = 2 * j + 1 < n_items;
-        load_item<NB, MODE>(opB, p, ld_tile, ld_set, has_b, kw, q, lane_col, tid);
-        advance(ld_tile, ld_set);
-        if (first) {
-            late_setup();
-            first_window();
+        for (int j = 1; j < pairs; ++j) {
+            load_item<NB, MODE>(opA, p, ld_tile, ld_set, true, kw, q, lane_col, tid);
+            advance(ld_tile, ld_set);
+            item_step(opB, false, no_hook);
+            const bool has_b = 2 * j + 1 < n_items;
+            load_item<NB, MODE>(opB, p, ld_tile, ld_set, has_b, kw, q, lane_col, tid);
+            advance(ld_tile, ld_set);
+            item_step(opA, !has_b, no_hook);
         }
-        item_step(opA, !has_b);
+        if ((n_items & 1) == 0) item_step(opB, true, no_hook);
+    } else {
+        // Several rows per pass, or per-lane block alphas: the register budget does not allow
+        // the first item a code path of its own (up to 300 bytes of spills per lane measured).  Everything is requested up front and the first iteration skips its
+        // first step at run time (opaque, which keeps the compiler from peeling it).
+#pragma clang loop unroll(disable)
+        for (int j = 0; j < pairs; ++j) {
+            int first = __builtin_amdgcn_readfirstlane(j == 0);
+            asm volatile("" : "+s"(first));
+            load_item<NB, MODE>(opA, p, ld_tile, ld_set, true, kw, q, lane_col, tid);
+            advance(ld_tile, ld_set);
+            if (!first) item_step(opB, false, no_hook);
+            const bool has_b = 2 * j + 1 < n_items;
+            load_item<NB, MODE>(opB, p, ld_tile, ld_set, has_b, kw, q, lane_col, tid);
+            advance(ld_tile, ld_set);
+            if (first) {
+                late_setup();
+                fetch_out(tile);
+                first_window();
+            }
+            item_step(opA, !has_b, no_hook);
+        }
+        if ((n_items & 1) == 0) item_step(opB, true, no_hook);
     }
-    if ((n_items & 1) == 0) item_step(opB, true);
 }
 
 // Flat workgroup index (relative to the problem) -> (range, row chunk), for launches
