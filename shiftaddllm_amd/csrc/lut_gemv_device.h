@@ -385,7 +385,8 @@ __device__ __forceinline__ float reduce_scatter_kw(const float (&acc)[4], int kw
 // are loaded once and used for all MROWS rows; tables are built per (item, row)
 // and double buffered.
 // EXTRA: the launch honours the split-RMSNorm fields of the problem (next_in, sumsq_*).
-template <int NB, int MODE, int MROWS, int XF = kXNone, bool EXTRA = false>
+// ALONE: the first item is requested on its own (see the main loop).
+template <int NB, int MODE, int MROWS, int XF = kXNone, bool EXTRA = false, bool ALONE = MROWS == 1 && !is_block(MODE)>
 __device__ __forceinline__ void gemv_range(const Problem &p, int range, int mchunk, float *lut)
 {
     static_assert(!(EXTRA || XF == kXNorm) || !is_staged(MODE), "the per-wave sums live in the alpha staging area");
@@ -718,7 +719,7 @@ __device__ __forceinline__ void gemv_range(const Problem &p, int range, int mchu
     int ld_tile = tile, ld_set = set;  // next item to request
     const int pairs = (n_items + 1) / 2;
     auto no_hook = []() {};
-    if constexpr (MROWS == 1 && !is_block(MODE)) {
+    if constexpr (ALONE) {
         load_item<NB, MODE, 1>(opA, p, ld_tile, ld_set, true, kw, q, lane_col, tid);
         __builtin_amdgcn_sched_barrier(0);
         late_setup();
@@ -742,8 +743,9 @@ __device__ __forceinline__ void gemv_range(const Problem &p, int range, int mchu
         }
         if ((n_items & 1) == 0) item_step(opB, true, no_hook);
     } else {
-        // Several rows per pass, or per-lane block alphas: the register budget does not allow
-        // the first item a code path of its own (up to 300 bytes of spills per lane measured).  Everything is requested up front and the first iteration skips its
+        // Several rows per pass, per-lane block alphas (the register budget does not allow the
+        // first item a code path of its own: up to 300 bytes of spills per lane measured), and
+        // grouped launches.  Everything is requested up front and the first iteration skips its
         // first step at run time (opaque, which keeps the compiler from peeling it).
 #pragma clang loop unroll(disable)
         for (int j = 0; j < pairs; ++j) {
@@ -786,6 +788,9 @@ lut_gemv_kernel(const Problem p)
 // Several row-wise problems in one launch.  Bit widths may differ between the
 // problems of a group.
 // XF: the input transform shared by all problems of the launch.
+// (Grouped launches keep the loop that requests two items up front: their ranges hold three
+// or four items, and requesting the second one late costs more than the first one gains:
+// q,k,v + o + gate,up + down of a 7B block 5.06 us per GEMV this way, 5.37 the other.)
 template <int XF>
 __global__ void __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4, 4)))
 lut_gemv_group_kernel(const Group g)
@@ -800,10 +805,10 @@ lut_gemv_group_kernel(const Group g)
     int range, m;
     decode_block(p, (int)blockIdx.x, range, m);
     switch (p.nb) {
-    case 1: gemv_range<1, kRowF16, 1, XF, true>(p, range, m, lut); break;
-    case 2: gemv_range<2, kRowF16, 1, XF, true>(p, range, m, lut); break;
-    case 3: gemv_range<3, kRowF16, 1, XF, true>(p, range, m, lut); break;
-    default: gemv_range<4, kRowF16, 1, XF, true>(p, range, m, lut); break;
+    case 1: gemv_range<1, kRowF16, 1, XF, true, false>(p, range, m, lut); break;
+    case 2: gemv_range<2, kRowF16, 1, XF, true, false>(p, range, m, lut); break;
+    case 3: gemv_range<3, kRowF16, 1, XF, true, false>(p, range, m, lut); break;
+    default: gemv_range<4, kRowF16, 1, XF, true, false>(p, range, m, lut); break;
     }
 }
 
