@@ -49,6 +49,14 @@ __device__ __forceinline__ float block_reduce(float v, float *red)
     return MAX ? fmaxf(fmaxf(a, b), fmaxf(c, d)) : (a + b) + (c + d);
 }
 
+// The value of another lane of the same row of 16, by a data-parallel-primitive move.
+template <int CTRL>
+__device__ __forceinline__ float dpp_lane(float v)
+{
+    const int vi = __builtin_bit_cast(int, v);
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(vi, vi, CTRL, 0xf, 0xf, false));
+}
+
 __device__ __forceinline__ void unpack8(const u32x4 &v, float f[8])
 {
     const uint32_t w[4] = {v.x, v.y, v.z, v.w};
@@ -223,9 +231,10 @@ attention_kernel(const __half *__restrict__ q, const __half *__restrict__ k, con
 }
 
 // The same for head_dim HD in {64, 128}, with the memory latency taken in
-// parallel: a thread fetches the whole key row of its position before using it,
-// and the value rows are walked by 256/(HD/8) position groups with four rows in
-// flight per thread.  Dynamic LDS: (3*HD + max_pos + 4 + (256/(HD/8))*HD) floats.
+// parallel and whole rows per load: thread (jg, ch) holds 16-byte chunk ch of key
+// and value rows jg, jg + 512/(HD/8), ... (sixteen of each in registers, requested
+// before the first barrier), a row's lanes meet by DPP moves for the scores.
+// Dynamic LDS: (3*HD + max_pos + 4 + (512/(HD/8))*HD) floats.
 template <int HD>
 __global__ void __launch_bounds__(kThreads)
 attention_hd_kernel(const __half *__restrict__ q, const __half *__restrict__ k, const __half *__restrict__ v,
@@ -269,51 +278,72 @@ attention_hd_kernel(const __half *__restrict__ q, const __half *__restrict__ k, 
             v_cache[(cache_row0 + pos) * HD + i] = vv;
         }
     }
-    // key and value rows of earlier positions do not depend on the above: fetch them
-    // before the barrier, so that the whole step costs one memory round trip
-    const bool first_pass_cached = tid < pos;
-    u32x4 row[kChunks];
-    if (first_pass_cached) {
-        const u32x4 *src = (const u32x4 *)(k_cache + (cache_row0 + tid) * HD);
-#pragma unroll
-        for (int c = 0; c < kChunks; ++c) row[c] = src[c];
-    }
-    constexpr int kValueRows = 16;  // value chunks per thread held in registers: 16 * kPosGroups positions
+    // Key and value rows of earlier positions do not depend on the above: fetch them
+    // before the barrier, so that the whole step costs one memory round trip.  Both are
+    // walked the same way: thread (jg, ch) takes 16-byte chunk ch of rows jg, jg +
+    // kPosGroups, ...: a wave's load covers whole rows (contiguous kilobytes), where a
+    // thread fetching "its" row chunk by chunk touches 64 cache lines per instruction.
+    constexpr int kRowsInRegs = 16;  // chunks per thread held in registers: 16 * kPosGroups positions
     const int jg = tid / kChunks, ch = tid % kChunks;
+    const u32x4 *kbase = (const u32x4 *)(k_cache + cache_row0 * HD) + ch;
     const u32x4 *vbase = (const u32x4 *)(v_cache + cache_row0 * HD) + ch;
-    u32x4 vrow[kValueRows];
+    u32x4 krow[kRowsInRegs], vrow[kRowsInRegs];
 #pragma unroll
-    for (int u = 0; u < kValueRows; ++u) {
+    for (int u = 0; u < kRowsInRegs; ++u) {
+        const int j = jg + u * kPosGroups;
+        krow[u] = (u32x4){0u, 0u, 0u, 0u};
+        if (j < pos) krow[u] = kbase[(size_t)j * kChunks];
+    }
+#pragma unroll
+    for (int u = 0; u < kRowsInRegs; ++u) {
         const int j = jg + u * kPosGroups;
         vrow[u] = (u32x4){0u, 0u, 0u, 0u};
         if (j < pos) vrow[u] = vbase[(size_t)j * kChunks];
     }
     __syncthreads();
 
+    // scores: each of a row's kChunks lanes multiplies its chunk, the lanes are summed
+    // inside their row of 16 (HD 128) or 8 (HD 64) lanes, lane 0 of the row keeps the score
     const float scale = rsqrtf((float)HD);
+    float qc[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) qc[i] = q_s[8 * ch + i];
+    auto row_sum = [](float v) {
+        v += dpp_lane<0xb1>(v);   // quad_perm [1,0,3,2]
+        v += dpp_lane<0x4e>(v);   // quad_perm [2,3,0,1]
+        v += dpp_lane<0x141>(v);  // row_half_mirror: the other quad of the 8
+        if (kChunks == 16) v += dpp_lane<0x140>(v);  // row_mirror: the other half of the 16
+        return v;
+    };
     float local_max = -INFINITY;
-    for (int j = tid; j <= pos; j += kThreads) {
+    auto score_row = [&](const u32x4 &kv, int j) {
+        float f[8];
+        unpack8(kv, f);
         float dot = 0.0f;
-        if (j == pos) {
 #pragma unroll
-            for (int i = 0; i < HD; ++i) dot = fmaf(q_s[i], k_s[i], dot);
-        } else {
-            if (j != tid) {
-                const u32x4 *src = (const u32x4 *)(k_cache + (cache_row0 + j) * HD);
-#pragma unroll
-                for (int c = 0; c < kChunks; ++c) row[c] = src[c];
-            }
-#pragma unroll
-            for (int c = 0; c < kChunks; ++c) {
-                float f[8];
-                unpack8(row[c], f);
-#pragma unroll
-                for (int i = 0; i < 8; ++i) dot = fmaf(q_s[8 * c + i], f[i], dot);
-            }
+        for (int i = 0; i < 8; ++i) dot = fmaf(qc[i], f[i], dot);
+        dot = row_sum(dot) * scale;
+        if (ch == 0 && j < pos) {
+            score[j] = dot;
+            local_max = fmaxf(local_max, dot);
         }
-        dot *= scale;
-        score[j] = dot;
-        local_max = fmaxf(local_max, dot);
+    };
+#pragma unroll
+    for (int u = 0; u < kRowsInRegs; ++u) score_row(krow[u], jg + u * kPosGroups);
+    for (int j0 = kRowsInRegs * kPosGroups; j0 < pos; j0 += kPosGroups) {  // longer contexts
+        const int j = j0 + jg;
+        score_row(kbase[(size_t)min(j, pos - 1) * kChunks], j);
+    }
+    {
+        // the new position's own key, still in LDS
+        float dot = 0.0f;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) dot = fmaf(qc[i], k_s[8 * ch + i], dot);
+        dot = row_sum(dot) * scale;
+        if (tid == 0) {
+            score[pos] = dot;
+            local_max = fmaxf(local_max, dot);
+        }
     }
     const float mx = block_reduce<true>(local_max, red);
     float local_sum = 0.0f;
@@ -328,7 +358,7 @@ attention_hd_kernel(const __half *__restrict__ q, const __half *__restrict__ k, 
 #pragma unroll
     for (int i = 0; i < 8; ++i) acc[i] = 0.0f;
 #pragma unroll
-    for (int u = 0; u < kValueRows; ++u) {
+    for (int u = 0; u < kRowsInRegs; ++u) {
         const int j = jg + u * kPosGroups;
         float f[8];
         unpack8(vrow[u], f);
@@ -336,7 +366,7 @@ attention_hd_kernel(const __half *__restrict__ q, const __half *__restrict__ k, 
 #pragma unroll
         for (int i = 0; i < 8; ++i) acc[i] = fmaf(pj, f[i], acc[i]);
     }
-    for (int j = jg + kValueRows * kPosGroups; j < pos; j += kPosGroups) {  // longer contexts
+    for (int j = jg + kRowsInRegs * kPosGroups; j < pos; j += kPosGroups) {  // longer contexts
         float f[8];
         unpack8(vbase[(size_t)j * kChunks], f);
         const float pj = score[j];
