@@ -14,6 +14,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <type_traits>
+
 #include "lutgemm_gfx950.h"
 #include "lutgemm_internal.h"
 
@@ -232,9 +234,13 @@ attention_kernel(const __half *__restrict__ q, const __half *__restrict__ k, con
 
 // The same for head_dim HD in {64, 128}, with the memory latency taken in
 // parallel and whole rows per load: thread (jg, ch) holds 16-byte chunk ch of key
-// and value rows jg, jg + 512/(HD/8), ... (sixteen of each in registers, requested
-// before the first barrier), a row's lanes meet by DPP moves for the scores.
-// Dynamic LDS: (3*HD + max_pos + 4 + (512/(HD/8))*HD) floats.
+// and value rows jg, jg + 256/(HD/8), ... (sixteen of each in registers, requested
+// before the first barrier; longer contexts go round in blocks of that size), a
+// row's lanes meet by DPP moves for the scores.  Each group of lanes keeps its own
+// running maximum, sum of exponentials and weighted value sum (the "online" form of
+// softmax), and the groups are merged once at the end: one barrier after the rotary
+// step and one before the merge, no pass over the scores in between.
+// Dynamic LDS: (3*HD + 2*(256/(HD/8)) + (256/(HD/8))*HD) floats.
 template <int HD>
 __global__ void __launch_bounds__(kThreads)
 attention_hd_kernel(const __half *__restrict__ q, const __half *__restrict__ k, const __half *__restrict__ v,
@@ -248,9 +254,9 @@ attention_hd_kernel(const __half *__restrict__ q, const __half *__restrict__ k, 
     float *q_s = lds;
     float *k_s = q_s + HD;
     float *v_s = k_s + HD;
-    float *score = v_s + HD;
-    float *red = score + max_pos;
-    float *part = red + 4;
+    float *grp_max = v_s + HD;
+    float *grp_sum = grp_max + kPosGroups;
+    float *part = grp_sum + kPosGroups;
 
     const int tid = threadIdx.x;
     const int b = blockIdx.x / H, h = blockIdx.x % H;
@@ -278,114 +284,121 @@ attention_hd_kernel(const __half *__restrict__ q, const __half *__restrict__ k, 
             v_cache[(cache_row0 + pos) * HD + i] = vv;
         }
     }
-    // Key and value rows of earlier positions do not depend on the above: fetch them
-    // before the barrier, so that the whole step costs one memory round trip.  Both are
-    // walked the same way: thread (jg, ch) takes 16-byte chunk ch of rows jg, jg +
-    // kPosGroups, ...: a wave's load covers whole rows (contiguous kilobytes), where a
-    // thread fetching "its" row chunk by chunk touches 64 cache lines per instruction.
-    constexpr int kRowsInRegs = 16;  // chunks per thread held in registers: 16 * kPosGroups positions
+    // Key and value rows of earlier positions do not depend on the above: the first block
+    // of them is fetched before the barrier, so that a step over a short context costs one
+    // memory round trip.  Both are walked the same way: thread (jg, ch) takes 16-byte chunk
+    // ch of rows jg, jg + kPosGroups, ...: a wave's load covers whole rows (contiguous
+    // kilobytes), where a thread fetching "its" row chunk by chunk touches 64 cache lines
+    // per instruction.
+    constexpr int kRowsInRegs = 16;  // rows per thread and block: a block is 16 * kPosGroups positions
+    constexpr int kBlock = kRowsInRegs * kPosGroups;
     const int jg = tid / kChunks, ch = tid % kChunks;
     const u32x4 *kbase = (const u32x4 *)(k_cache + cache_row0 * HD) + ch;
     const u32x4 *vbase = (const u32x4 *)(v_cache + cache_row0 * HD) + ch;
     u32x4 krow[kRowsInRegs], vrow[kRowsInRegs];
+    auto fetch_block = [&](int j0) {
 #pragma unroll
-    for (int u = 0; u < kRowsInRegs; ++u) {
-        const int j = jg + u * kPosGroups;
-        krow[u] = (u32x4){0u, 0u, 0u, 0u};
-        if (j < pos) krow[u] = kbase[(size_t)j * kChunks];
-    }
+        for (int u = 0; u < kRowsInRegs; ++u) {
+            const int j = j0 + jg + u * kPosGroups;
+            krow[u] = (u32x4){0u, 0u, 0u, 0u};
+            if (j < pos) krow[u] = kbase[(size_t)j * kChunks];
+        }
 #pragma unroll
-    for (int u = 0; u < kRowsInRegs; ++u) {
-        const int j = jg + u * kPosGroups;
-        vrow[u] = (u32x4){0u, 0u, 0u, 0u};
-        if (j < pos) vrow[u] = vbase[(size_t)j * kChunks];
-    }
+        for (int u = 0; u < kRowsInRegs; ++u) {
+            const int j = j0 + jg + u * kPosGroups;
+            vrow[u] = (u32x4){0u, 0u, 0u, 0u};
+            if (j < pos) vrow[u] = vbase[(size_t)j * kChunks];
+        }
+    };
+    fetch_block(0);
     __syncthreads();
 
-    // scores: each of a row's kChunks lanes multiplies its chunk, the lanes are summed
-    // inside their row of 16 (HD 128) or 8 (HD 64) lanes, lane 0 of the row keeps the score
+    // a row's kChunks lanes multiply their chunks and are summed inside their row of 16
+    // (HD 128) or 8 (HD 64) lanes: every lane of the row ends up with the score
     const float scale = rsqrtf((float)HD);
     float qc[8];
 #pragma unroll
     for (int i = 0; i < 8; ++i) qc[i] = q_s[8 * ch + i];
-    auto row_sum = [](float v) {
-        v += dpp_lane<0xb1>(v);   // quad_perm [1,0,3,2]
-        v += dpp_lane<0x4e>(v);   // quad_perm [2,3,0,1]
-        v += dpp_lane<0x141>(v);  // row_half_mirror: the other quad of the 8
-        if (kChunks == 16) v += dpp_lane<0x140>(v);  // row_mirror: the other half of the 16
-        return v;
+    auto row_sum = [](float x) {
+        x += dpp_lane<0xb1>(x);   // quad_perm [1,0,3,2]
+        x += dpp_lane<0x4e>(x);   // quad_perm [2,3,0,1]
+        x += dpp_lane<0x141>(x);  // row_half_mirror: the other quad of the 8
+        if (kChunks == 16) x += dpp_lane<0x140>(x);  // row_mirror: the other half of the 16
+        return x;
     };
-    float local_max = -INFINITY;
-    auto score_row = [&](const u32x4 &kv, int j) {
-        float f[8];
-        unpack8(kv, f);
-        float dot = 0.0f;
+    // running state of this thread's rows: maximum score, sum of exp(score - maximum), and
+    // the same weights applied to the value chunks
+    float run_max = -INFINITY, run_sum = 0.0f, acc[8];
 #pragma unroll
-        for (int i = 0; i < 8; ++i) dot = fmaf(qc[i], f[i], dot);
-        dot = row_sum(dot) * scale;
-        if (ch == 0 && j < pos) {
-            score[j] = dot;
-            local_max = fmaxf(local_max, dot);
+    for (int i = 0; i < 8; ++i) acc[i] = 0.0f;
+    auto fold = [&](const float *sc, auto &&value_of, auto row_count) {
+        constexpr int rows = decltype(row_count)::value;
+        float blk_max = run_max;
+#pragma unroll
+        for (int u = 0; u < rows; ++u) blk_max = fmaxf(blk_max, sc[u]);
+        if (blk_max == -INFINITY) return;  // nothing valid so far (uniform over the row's lanes)
+        const float keep = __expf(run_max - blk_max);  // 0 when nothing was held before
+        run_sum *= keep;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) acc[i] *= keep;
+#pragma unroll
+        for (int u = 0; u < rows; ++u) {
+            const float pj = __expf(sc[u] - blk_max);  // 0 for a masked row
+            run_sum += pj;
+            float f[8];
+            value_of(u, f);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) acc[i] = fmaf(pj, f[i], acc[i]);
         }
+        run_max = blk_max;
     };
+    for (int j0 = 0; j0 < pos; j0 += kBlock) {
+        if (j0) fetch_block(j0);
+        float sc[kRowsInRegs];
 #pragma unroll
-    for (int u = 0; u < kRowsInRegs; ++u) score_row(krow[u], jg + u * kPosGroups);
-    for (int j0 = kRowsInRegs * kPosGroups; j0 < pos; j0 += kPosGroups) {  // longer contexts
-        const int j = j0 + jg;
-        score_row(kbase[(size_t)min(j, pos - 1) * kChunks], j);
+        for (int u = 0; u < kRowsInRegs; ++u) {
+            float f[8];
+            unpack8(krow[u], f);
+            float dot = 0.0f;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) dot = fmaf(qc[i], f[i], dot);
+            dot = row_sum(dot) * scale;
+            sc[u] = j0 + jg + u * kPosGroups < pos ? dot : -INFINITY;
+        }
+        fold(sc, [&](int u, float *f) { unpack8(vrow[u], f); }, std::integral_constant<int, kRowsInRegs>());
     }
-    {
-        // the new position's own key, still in LDS
+    if (jg == 0) {
+        // the new position's own key and value, still in LDS
         float dot = 0.0f;
 #pragma unroll
         for (int i = 0; i < 8; ++i) dot = fmaf(qc[i], k_s[8 * ch + i], dot);
-        dot = row_sum(dot) * scale;
-        if (tid == 0) {
-            score[pos] = dot;
-            local_max = fmaxf(local_max, dot);
-        }
-    }
-    const float mx = block_reduce<true>(local_max, red);
-    float local_sum = 0.0f;
-    for (int j = tid; j <= pos; j += kThreads) {
-        const float e = __expf(score[j] - mx);
-        score[j] = e;
-        local_sum += e;
-    }
-    const float inv = 1.0f / block_reduce<false>(local_sum, red);  // its barriers also publish score[]
-
-    float acc[8];
+        const float own = row_sum(dot) * scale;
+        fold(&own, [&](int, float *f) {
 #pragma unroll
-    for (int i = 0; i < 8; ++i) acc[i] = 0.0f;
-#pragma unroll
-    for (int u = 0; u < kRowsInRegs; ++u) {
-        const int j = jg + u * kPosGroups;
-        float f[8];
-        unpack8(vrow[u], f);
-        const float pj = j < pos ? score[j] : 0.0f;
-#pragma unroll
-        for (int i = 0; i < 8; ++i) acc[i] = fmaf(pj, f[i], acc[i]);
-    }
-    for (int j = jg + kRowsInRegs * kPosGroups; j < pos; j += kPosGroups) {  // longer contexts
-        float f[8];
-        unpack8(vbase[(size_t)j * kChunks], f);
-        const float pj = score[j];
-#pragma unroll
-        for (int i = 0; i < 8; ++i) acc[i] = fmaf(pj, f[i], acc[i]);
-    }
-    if (jg == 0) {
-        const float pj = score[pos];
-#pragma unroll
-        for (int i = 0; i < 8; ++i) acc[i] = fmaf(pj, v_s[8 * ch + i], acc[i]);
+            for (int i = 0; i < 8; ++i) f[i] = v_s[8 * ch + i];
+        }, std::integral_constant<int, 1>());
     }
 #pragma unroll
     for (int i = 0; i < 8; ++i) part[jg * HD + 8 * ch + i] = acc[i];
+    if (ch == 0) {
+        grp_max[jg] = run_max;
+        grp_sum[jg] = run_sum;
+    }
     __syncthreads();
     if (tid < HD) {
-        float sum = 0.0f;
+        // merge the groups: weights exp(group maximum - overall maximum); group 0 always holds
+        // the new position, so the overall maximum is finite
+        float mx = -INFINITY;
+#pragma unroll
+        for (int g = 0; g < kPosGroups; ++g) mx = fmaxf(mx, grp_max[g]);
+        float sum = 0.0f, total = 0.0f;
 #pragma unroll 8
-        for (int g = 0; g < kPosGroups; ++g) sum += part[g * HD + tid];
-        out[((size_t)b * H + h) * HD + tid] = __float2half_rn(sum * inv);
+        for (int g = 0; g < kPosGroups; ++g) {
+            const float w = __expf(grp_max[g] - mx);  // 0 for a group without rows
+            total = fmaf(grp_sum[g], w, total);
+            sum = fmaf(part[g * HD + tid], w, sum);
+        }
+        out[((size_t)b * H + h) * HD + tid] = __float2half_rn(sum / total);
     }
 }
 
@@ -450,8 +463,7 @@ int lutgemm_decode_attention_f16(const void *q, const void *k, const void *v, co
     if (!aligned16(k_cache) || !aligned16(v_cache)) return LUTGEMM_EALIGN;
     if (head_dim == 64 || head_dim == 128) {
         const int pos_groups = kThreads / (head_dim / 8);
-        const size_t lds_hd =
-            sizeof(float) * ((size_t)3 * head_dim + max_positions + 4 + (size_t)pos_groups * head_dim);
+        const size_t lds_hd = sizeof(float) * ((size_t)3 * head_dim + 2 * pos_groups + (size_t)pos_groups * head_dim);
         if (head_dim == 128)
             hipLaunchKernelGGL(attention_hd_kernel<128>, dim3((unsigned)(batch * heads)), dim3(kThreads), lds_hd,
                                (hipStream_t)stream, (const __half *)q, (const __half *)k, (const __half *)v,
