@@ -601,10 +601,11 @@ def main():
                                 f"random.Random(0) ({counts[2]}x2-bit, {counts[3]}x3-bit, {counts[4]}x4-bit), "
                                 "group 128, 128 prompt tokens fed one by one then 128 greedy tokens, one "
                                 "HIP-graph replay + sync per token; q/k/v and gate/up as grouped launches; "
-                                "RMSNorm split over the GEMV that completes the residual row and the GEMVs that "
-                                "read it (no norm launches inside the stack); rotary + KV append + attention as one "
-                                "HIP kernel; batch 1: look-up kernel, SiLU*up folded into the down_proj GEMV "
-                                "(5 launches per block); batch 8: matrix-core kernel, SiLU*up as a HIP kernel "
+                                "no norm launches inside the stack; rotary + KV append + attention as one "
+                                "HIP kernel; batch 1: look-up kernel, RMSNorm folded into the q/k/v and gate/up "
+                                "launches, SiLU*up folded into the down_proj GEMV (5 launches per block); "
+                                "batch 8: matrix-core kernel, RMSNorm split over the GEMV that completes the "
+                                "residual row and the GEMVs that read it, SiLU*up as a HIP kernel "
                                 "(6 launches per block); embedding gather and fp16 lm_head in torch")
 
     traffic = None

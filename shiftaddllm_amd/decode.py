@@ -103,9 +103,10 @@ class LutDecoder(nn.Module):
         if glue not in ("hip", "torch"):
             raise ValueError(f"glue must be 'hip' or 'torch', got {glue!r}")
         self.cfg, self.batch, self.fuse, self.glue = cfg, batch, fuse_launches, glue
-        # RMSNorm inside the q,k,v and gate,up GEMVs instead of a kernel of its own (every workgroup
-        # re-reads the row to form its RMS: measured no faster than the separate kernel)
-        self.fold_norm = False
+        # One or two sequences: RMSNorm inside the q,k,v and gate,up GEMVs (every workgroup re-reads
+        # the row to form its RMS and scales its finished sums; the look-up kernel only).  Measured
+        # against the split below on the 7B decoder at one sequence: 1.535 vs 1.572 ms per token.
+        self.fold_norm = fuse_launches and batch <= 2
         # RMSNorm split over the GEMV that completes the residual row (it leaves x * norm weight and
         # the row's sums of squares) and the GEMVs that read it (they scale their sums): no norm
         # launches inside the stack, for any batch size

@@ -58,6 +58,8 @@ def _rope(t, cos, sin):
     (2, 8, 2, 128, 700, (0, 300, 699)),        # more keys than threads in a workgroup
     (1, 4, 4, 96, 40, (0, 17, 39)),            # the generic head-dim path
     (3, 6, 3, 64, 520, (519,)),
+    (1, 2, 2, 128, 1100, (256, 257, 512, 1099)),   # either side of the 256-position blocks the kernel walks in
+    (1, 2, 1, 64, 1030, (511, 512, 513, 1029)),    # (512 positions a block at this head size)
 ])
 def test_attention_step(gpu_device, B, H, KV, hd, max_pos, positions):
     lib = native.cabi()
