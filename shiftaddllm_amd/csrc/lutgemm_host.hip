@@ -278,15 +278,13 @@ bool mfma_eligible(const Problem &p, int mode)
     return p.M == 2 && mfma_min_rows() == 3 && (long)p.N * (p.K / 8) * p.nb <= (32l << 20);
 }
 
-// K-steps are split 8 ways inside a workgroup already; across workgroups only as
-// far as needed to reach `want_blocks`.
-void plan_mfma(Problem &p, int mt, long want_blocks)
+// K-steps are split 8 ways inside a workgroup already; across workgroups `want` ways
+// at most (whole rounds of eight steps per slice).
+void plan_mfma(Problem &p, int mt, long want)
 {
     p.n_tiles = (p.N + kMfmaTileCols - 1) / kMfmaTileCols;
     p.mchunks = (p.M + 16 * mt - 1) / (16 * mt);
     p.nsets = p.K / kMfmaStepK;  // K-steps
-    long want = want_blocks / ((long)p.n_tiles * p.mchunks);
-    if (want < 1) want = 1;
     if (want > p.nsets / kMfmaWaves) want = p.nsets / kMfmaWaves;
     if (want < 1) want = 1;
     if (want > kMaxContrib) want = kMaxContrib;
@@ -296,20 +294,73 @@ void plan_mfma(Problem &p, int mt, long want_blocks)
     p.n_blocks = p.n_tiles * p.ksplit * p.mchunks;
 }
 
-// Workgroups wanted per launch: two per CU for the 16-row tile (its register count
-// lets two be resident), one per CU for the 32-row tile.  Measured, 8192x8192x2:
-// 16 rows 16.9 us at 256 and 15.1 at 512; 32 rows 36.4 at 256 and 40.0 at 512 (4 bits).
-int mfma_blocks(int mt)
+// Workgroups wanted per launch of the 32-row tile: one per CU (its register count allows
+// no second one).  Measured, 8192x8192x4: 36.4 us at 256 and 40.0 at 512.
+int mfma_blocks_override()
 {
     static const int v = env_int("LUTGEMM_MFMA_BLOCKS", 0);
-    if (v > 0) return v;
-    return mt == 1 ? 512 : 256;
+    return v;
+}
+
+// K-slices per tile for the problems of one launch (all get the same number, each up to
+// its own limit).
+//   32-row tile: as many as reach one workgroup per CU.
+//   16-row tile: the kernel is bound by the vector ALU work of expanding sign bits, two
+//   workgroups share a CU, and the launch ends when the busiest CU does.  With w =
+//   ceil(workgroups / 256) workgroups on that CU and R rounds (one K-step per wave, about
+//   2.2 us at three bit planes) per workgroup, the slice count that minimises
+//       w * R  +  0.18 * w  +  0.9 * max(0, w - 2)
+//   is taken, the smaller one on ties: a workgroup's start and hand-over cost a fifth of a
+//   round, and one that has to wait for a slot on its CU most of a round.  A lone workgroup
+//   of four or more rounds hides its loads badly when there are many of them (more than
+//   eight activation rows, or nine CUs in ten busy) and is charged 12 % more.  Fitted to
+//   launches at 4 and 16 rows (us, slices -> time): 8192x8192x4: 2 -> 17.9, 4 -> 16.7;
+//   11008x4096x3: 1 -> 13.0, 2 -> 13.4 (16 rows: 16.7, 14.9); 22016x4096x3: 1 -> 21.4, 2 -> 18.3;
+//   28672x8192x2: 1 -> 28.1, 4 -> 32.5; 5120x13824x3: 3 -> 16.2, 5 -> 18.4.
+int mfma_slices(const Group &g, int mt)
+{
+    constexpr long kCUs = 256;
+    long tiles = 0;
+    int max_rounds = 1, rows = 0;
+    for (int i = 0; i < g.count; ++i) {
+        const Problem &p = g.p[i];
+        tiles += (long)((p.N + kMfmaTileCols - 1) / kMfmaTileCols) * ((p.M + 16 * mt - 1) / (16 * mt));
+        const int rounds = p.K / kMfmaStepK / kMfmaWaves;
+        if (rounds > max_rounds) max_rounds = rounds;
+        if (p.M > rows) rows = p.M;
+    }
+    if (max_rounds > kMaxContrib) max_rounds = kMaxContrib;
+    if (const int blocks = mfma_blocks_override()) return (int)(blocks / tiles > 1 ? blocks / tiles : 1);
+    if (mt != 1) return (int)(kCUs / tiles > 1 ? kCUs / tiles : 1);
+    int best = 1;
+    double best_cost = 0.0;
+    for (int ks = 1; ks <= max_rounds; ++ks) {
+        long wgs = 0;
+        int rounds = 0;
+        for (int i = 0; i < g.count; ++i) {
+            Problem q = g.p[i];
+            plan_mfma(q, mt, ks);
+            wgs += q.n_blocks;
+            if (q.sets_per_split / kMfmaWaves > rounds) rounds = q.sets_per_split / kMfmaWaves;
+        }
+        const long w = (wgs + kCUs - 1) / kCUs;
+        double cost = (double)w * rounds + 0.18 * (double)w + 0.9 * (double)(w > 2 ? w - 2 : 0);
+        if (w == 1 && rounds >= 4 && (rows > 8 || wgs * 10 > kCUs * 9)) cost *= 1.12;
+        if (ks == 1 || cost < best_cost * 0.999) {
+            best = ks;
+            best_cost = cost;
+        }
+    }
+    return best;
 }
 
 int run_mfma(Problem &p, const Accum &acc)
 {
     const int mt = p.M > 16 ? 2 : 1;
-    plan_mfma(p, mt, mfma_blocks(mt));
+    Group one{};
+    one.count = 1;
+    one.p[0] = p;
+    plan_mfma(p, mt, mfma_slices(one, mt));
     if (p.ksplit > 1) {
         int rc = accum_words(acc, (size_t)p.M * p.N, &p.accum);
         if (rc != LUTGEMM_OK) return rc;
@@ -323,18 +374,14 @@ int run_mfma(Problem &p, const Accum &acc)
 int run_mfma_group(Group &g, const Accum &acc)
 {
     const int mt = g.p[0].M > 16 ? 2 : 1;
-    long total_bytes = 0;
     size_t words = 0;
-    for (int i = 0; i < g.count; ++i) {
-        total_bytes += (long)g.p[i].N * (g.p[i].K / 8) * g.p[i].nb;
-        words += (size_t)g.p[i].M * g.p[i].N;
-    }
+    for (int i = 0; i < g.count; ++i) words += (size_t)g.p[i].M * g.p[i].N;
+    const int slices = mfma_slices(g, mt);
     int begin = 0;
     bool any_split = false;
     for (int i = 0; i < g.count; ++i) {
         Problem &p = g.p[i];
-        const long mine = (long)p.N * (p.K / 8) * p.nb;
-        plan_mfma(p, mt, (long)mfma_blocks(mt) * mine / (total_bytes > 0 ? total_bytes : 1));
+        plan_mfma(p, mt, slices);
         if (p.n_blocks > begin) begin = p.n_blocks;  // grid.x: the largest problem's workgroups
         any_split = any_split || p.ksplit > 1;
     }
