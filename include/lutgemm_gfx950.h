@@ -20,7 +20,11 @@
  *           the caller pre-fills out with the bias or zeros
  *           (mv_fp16_bias.hpp:101,216,324,491,577; lut_gemm/quant.py:46).
  *           Unlike the reference's fp16 atomics the sum is formed in fp32 and
- *           rounded to fp16 once, and it is deterministic.
+ *           rounded to fp16 once, and it is deterministic.  (Two to four rows
+ *           of a per-column-alpha problem on the table look-up kernel share
+ *           tables whose entries are fp16, like the reference's
+ *           (mv_fp16_bias.hpp:342-380): one more fp16 rounding per eight
+ *           inputs, output error about 3e-4 relative instead of 2e-4.)
  *           A NaN input gives NaN and an infinite input gives an infinity
  *           or NaN in every output it reaches, whatever the launch plan
  *           (partial sums beyond +-65536 count as infinite).

@@ -284,6 +284,62 @@ __device__ __forceinline__ void build_tables(const u32x4 &xraw, float *lut, int 
     }
 }
 
+// The same for two activation rows at once: an entry is the pair (row a, row b) as two
+// fp16 halves of one word, so that one look-up serves both rows.  The sums are formed
+// in fp32 like the single-row tables and rounded once when packed (the reference's own
+// tables are fp16 sums of fp16 values, mv_fp16_bias.hpp:342-380).
+__device__ __forceinline__ uint32_t pack_entry(float a, float b)
+{
+    const __half2 h = __floats2half2_rn(a, b);
+    return __builtin_bit_cast(uint32_t, h);
+}
+
+__device__ __forceinline__ void build_tables_pair(const u32x4 &xa, const u32x4 &xb, float *lut, int buf, int tb, int eb)
+{
+    float a2[8], b2[8];  // 2 * x of either row
+    float base_a = 0.0f, base_b = 0.0f;
+    const uint32_t ra[4] = {xa.x, xa.y, xa.z, xa.w};
+    const uint32_t rb[4] = {xb.x, xb.y, xb.z, xb.w};
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const float alo = half_bits_to_float(ra[j] & 0xffffu), ahi = half_bits_to_float(ra[j] >> 16);
+        const float blo = half_bits_to_float(rb[j] & 0xffffu), bhi = half_bits_to_float(rb[j] >> 16);
+        a2[2 * j] = alo + alo;
+        a2[2 * j + 1] = ahi + ahi;
+        b2[2 * j] = blo + blo;
+        b2[2 * j + 1] = bhi + bhi;
+        base_a -= alo + ahi;
+        base_b -= blo + bhi;
+    }
+    float top_a = base_a, top_b = base_b;
+#pragma unroll
+    for (int j = 4; j < 8; ++j)
+        if ((eb >> (j - 4)) & 1) {
+            top_a += a2[j];
+            top_b += b2[j];
+        }
+    uint32_t *col = (uint32_t *)lut + (eb * 16) * kEntryStride + buf * kTables + tb;
+#pragma unroll
+    for (int sb = 0; sb < 2; ++sb) {
+        float va = top_a, vb = top_b;
+        if (sb & 1) {
+            va += a2[3];
+            vb += b2[3];
+        }
+        unsigned gray = 0;
+        col[(sb * 8) * kEntryStride] = pack_entry(va, vb);
+#pragma unroll
+        for (int i = 1; i < 8; ++i) {
+            const int bit = __builtin_ctz(i);
+            gray ^= 1u << bit;
+            const bool up = (gray >> bit) & 1u;
+            va += up ? a2[bit] : -a2[bit];
+            vb += up ? b2[bit] : -b2[bit];
+            col[(sb * 8 + gray) * kEntryStride] = pack_entry(va, vb);
+        }
+    }
+}
+
 // This lane's look-ups of one item against the table buffer `lane_off` selects.
 // lane_off: byte j = 4*(bank of the table used at step j + 32*buffer).
 // sel[j]  : v_perm_b32 selector putting byte (j+q)&3 of the sign word into
@@ -356,6 +412,70 @@ __device__ __forceinline__ void lookup_item(const ItemOperands<NB, MODE> &cur, c
     }
 }
 
+// The same against pair tables (build_tables_pair): one look-up, two rows.  Row-wise and
+// uniform alphas only.
+template <int NB, int MODE>
+__device__ __forceinline__ void lookup_item_pair(const ItemOperands<NB, MODE> &cur, const float *lut, float (&acc_a)[4],
+                                                 float (&acc_b)[4], uint32_t lane_off, const uint32_t (&sel)[4])
+{
+    static_assert(MODE == kRowF16 || MODE == kUniformF16, "pair tables: per-column alphas only");
+    const char *lut_bytes = (const char *)lut;
+    constexpr int kUnits = 2 * NB;
+    uint32_t val[2][8];
+    auto lo = [](uint32_t w) { return half_bits_to_float(w & 0xffffu); };
+    auto hi = [](uint32_t w) { return half_bits_to_float(w >> 16); };
+    auto issue = [&](int u, uint32_t (&v)[8]) {
+        const int b = u >> 1, i0 = (u & 1) * 2;
+        const uint32_t w4[4] = {cur.w[b].x, cur.w[b].y, cur.w[b].z, cur.w[b].w};
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                v[4 * i + j] = *(const uint32_t *)(lut_bytes + __builtin_amdgcn_perm(w4[i0 + i], lane_off, sel[j]));
+    };
+    auto retire = [&](int u, const uint32_t (&v)[8]) {
+        const int b = u >> 1, i0 = (u & 1) * 2;
+        [[maybe_unused]] const uint32_t ar = (u & 1) ? cur.a_row[b].y : cur.a_row[b].x;
+        [[maybe_unused]] const uint32_t au = (u & 1) ? cur.a_uni.y : cur.a_uni.x;
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            float a;
+            if constexpr (MODE == kRowF16)
+                a = half_bits_to_float((ar >> (16 * i)) & 0xffffu);
+            else
+                a = half_bits_to_float((au >> (16 * i)) & 0xffffu) * (1.0f / (float)(2 << b));
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                acc_a[i0 + i] = fmaf(lo(v[4 * i + j]), a, acc_a[i0 + i]);
+                acc_b[i0 + i] = fmaf(hi(v[4 * i + j]), a, acc_b[i0 + i]);
+            }
+        }
+    };
+    issue(0, val[0]);
+    if constexpr (MODE == kUniformF16) {
+        // sums of the lane's 32 inputs = entry 255 of its four tables
+        float sum_a = 0.0f, sum_b = 0.0f;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const uint32_t e = *(const uint32_t *)(lut_bytes + 255 * 4 * kEntryStride + ((lane_off >> (8 * j)) & 255u));
+            sum_a += lo(e);
+            sum_b += hi(e);
+        }
+        const uint32_t rq[2] = {cur.q_uni.x, cur.q_uni.y};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const float qb = half_bits_to_float((rq[i >> 1] >> (16 * (i & 1))) & 0xffffu);
+            acc_a[i] = fmaf(qb, sum_a, acc_a[i]);
+            acc_b[i] = fmaf(qb, sum_b, acc_b[i]);
+        }
+    }
+#pragma unroll
+    for (int u = 0; u < kUnits; ++u) {
+        if (u + 1 < kUnits) issue(u + 1, val[(u + 1) & 1]);
+        retire(u, val[u & 1]);
+    }
+}
+
 // ds_swizzle in bit-mask mode: the value of lane (l ^ XOR) within each group of 32.
 template <int XOR>
 __device__ __forceinline__ float swizzle_xor(float v)
@@ -386,9 +506,13 @@ __device__ __forceinline__ float reduce_scatter_kw(const float (&acc)[4], int kw
 // and double buffered.
 // EXTRA: the launch honours the split-RMSNorm fields of the problem (next_in, sumsq_*).
 // ALONE: the first item is requested on its own (see the main loop).
-template <int NB, int MODE, int MROWS, int XF = kXNone, bool EXTRA = false, bool ALONE = MROWS == 1 && !is_block(MODE)>
+// PAIR: rows are taken two at a time through pair tables (fp16 entries; MROWS even,
+//       per-column alphas).
+template <int NB, int MODE, int MROWS, int XF = kXNone, bool EXTRA = false, bool ALONE = MROWS == 1 && !is_block(MODE),
+          bool PAIR = false>
 __device__ __forceinline__ void gemv_range(const Problem &p, int range, int mchunk, float *lut)
 {
+    static_assert(!PAIR || (MROWS % 2 == 0 && (MODE == kRowF16 || MODE == kUniformF16)), "pair tables: even row count, per-column alphas");
     static_assert(!(EXTRA || XF == kXNorm) || !is_staged(MODE), "the per-wave sums live in the alpha staging area");
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -447,7 +571,7 @@ __device__ __forceinline__ void gemv_range(const Problem &p, int range, int mchu
     const int set0 = set, n_items = rem;
     float *window = stage + kStageDwords;
     const WindowChunk w0 = fetch_window<MROWS, XF>(p, m0, set0, 0, n_items, tid);
-    constexpr bool kDirectFirst = XF == kXNone;
+    constexpr bool kDirectFirst = XF == kXNone && !PAIR;
     // Without an input transform the tables of the first item (row 0) are built straight
     // from a second request for this thread's own chunk, so that nothing but that chunk
     // stands between the start of the kernel and the first table.
@@ -657,8 +781,26 @@ __device__ __forceinline__ void gemv_range(const Problem &p, int range, int mchu
             store_window<MROWS, XF>(w, window, tid);
             __syncthreads();
         }
+        if constexpr (PAIR) {
 #pragma unroll
-        for (int r = 0; r < MROWS; ++r) {
+            for (int rp = 0; rp < MROWS / 2; ++rp) {
+                const u32x4 xa = *(const u32x4 *)(window + 4 * (((2 * rp) * kSlots + slot) * kTables + tb));
+                const u32x4 xb = *(const u32x4 *)(window + 4 * (((2 * rp + 1) * kSlots + slot) * kTables + tb));
+                build_tables_pair(xa, xb, lut, buf, tb, eb);
+                __syncthreads();
+                if (rp == 0) {
+                    __builtin_amdgcn_sched_barrier(0);
+                    after_first_barrier();
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+                asm volatile("" : "+v"(lane_off));
+                lookup_item_pair<NB, MODE>(ops, lut, acc[2 * rp], acc[2 * rp + 1], lane_off, sel);
+                buf ^= 1;
+                lane_off ^= kFlip;
+            }
+        }
+#pragma unroll
+        for (int r = 0; r < (PAIR ? 0 : MROWS); ++r) {
             u32x4 xr = x0;
             if (!kDirectFirst || r > 0 || rel > 0) {
                 xr = *(const u32x4 *)(window + 4 * ((r * kSlots + slot) * kTables + tb));
@@ -777,12 +919,13 @@ __device__ __forceinline__ void decode_block(const Problem &p, int local, int &r
 }
 
 // (at most 128 registers, so that two workgroups share a CU)
-template <int NB, int MODE, int MROWS>
+template <int NB, int MODE, int MROWS, bool PAIR = false>
 __global__ void __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4, 4)))
 lut_gemv_kernel(const Problem p)
 {
     __shared__ __attribute__((aligned(16))) float lut[kLutDwords + kStageDwords + kWindowDwords];
-    gemv_range<NB, MODE, MROWS>(p, (int)blockIdx.x, (int)blockIdx.y, lut);  // grid = (ranges, row chunks)
+    // grid = (ranges, row chunks)
+    gemv_range<NB, MODE, MROWS, kXNone, false, MROWS == 1 && !is_block(MODE), PAIR>(p, (int)blockIdx.x, (int)blockIdx.y, lut);
 }
 
 // Several row-wise problems in one launch.  Bit widths may differ between the

@@ -1,16 +1,31 @@
 // Look-up kernel instances: row-wise alpha (lut_gemm/mv_fp16_bias.hpp:498-579 of the
 // ShiftAddLLM checkout) and uniform mode with q_bias (mv_fp16_bias.hpp:8-103).
+#include <stdlib.h>
+
 #include "lut_gemv_device.h"
 #include "lutgemm_launch.h"
 
 namespace lutgemm {
 namespace {
 
+// Rows are taken two at a time through tables whose entries hold both rows as fp16
+// halves; LUTGEMM_PAIR_TABLES=0 keeps one fp32 table set per row.
+bool pair_tables_enabled()
+{
+    const char *v = getenv("LUTGEMM_PAIR_TABLES");
+    return !(v && *v == '0');
+}
+
 template <int NB, int MODE>
 hipError_t launch_nb(const Problem &p, int mrows, hipStream_t stream)
 {
+    static const bool pair_tables = pair_tables_enabled();
     const dim3 grid((unsigned)p.wgs_per_chunk, (unsigned)p.mchunks), block(kThreads);
-    if (mrows == 4)
+    if (mrows == 4 && pair_tables)
+        hipLaunchKernelGGL((lut_gemv_kernel<NB, MODE, 4, true>), grid, block, 0, stream, p);
+    else if (mrows == 2 && pair_tables)
+        hipLaunchKernelGGL((lut_gemv_kernel<NB, MODE, 2, true>), grid, block, 0, stream, p);
+    else if (mrows == 4)
         hipLaunchKernelGGL((lut_gemv_kernel<NB, MODE, 4>), grid, block, 0, stream, p);
     else if (mrows == 2)
         hipLaunchKernelGGL((lut_gemv_kernel<NB, MODE, 2>), grid, block, 0, stream, p);

@@ -272,10 +272,11 @@ bool mfma_eligible(const Problem &p, int mode)
     if (!(mode == kRowF16 && p.K % kMfmaStepK == 0 && p.group_words % 4 == 0 && p.N % 16 == 0 && p.N >= 16))
         return false;
     if (p.M >= mfma_min_rows()) return true;
-    // two rows: the look-up kernel wins only where the sign stream is long enough to
-    // hide its per-row work (measured, look-up vs matrix core: 4096x4096x3 13.4 us vs
-    // 7.4; 8192x8192x4 21.8 vs 19.9; 28672x8192x2 about 30 vs 38.9; 28672x8192x4 46 vs 62)
-    return p.M == 2 && mfma_min_rows() == 3 && (long)p.N * (p.K / 8) * p.nb <= (32l << 20);
+    // two rows: the look-up kernel (one table set for both rows, fp16 entry pairs) wins from
+    // about 12 MB of sign words on (measured, look-up vs matrix core: 4096x4096x3 7.3 us vs 6.4;
+    // 11008x4096x2 10.5 vs 9.6; 5120x5120x4 9.8 vs 10.5; 11008x4096x3 11.9 vs 12.8; 8192x8192x4
+    // 14.2 vs 16.6; 28672x8192x4 34.7 vs 52)
+    return p.M == 2 && mfma_min_rows() == 3 && (long)p.N * (p.K / 8) * p.nb <= (12l << 20);
 }
 
 // K-steps are split 8 ways inside a workgroup already; across workgroups `want` ways

@@ -20,6 +20,7 @@ pytestmark = pytest.mark.gpu
 REL_L2_BAR = 2e-3          # relative L2 error bound on the fp16 output
 MAX_ABS_BAR = 1e-2         # max |dy| / max |y_ref|
 TIGHT = 0.1                # our own margin inside those bars
+PAIR_TABLES = 0.25         # the same for rows that share fp16-pair tables (see _rows_margin)
 
 
 def _stream():
@@ -104,7 +105,33 @@ def test_rowwise_ragged_shapes(gpu_device, N, K, nb, gs, M):
     p = workload.make_rowwise_problem(N, K, nb=nb, group_size=gs, M=M, seed=N + K + nb, quantize=False)
     want, _ = orc.gemv_rowwise_c(p.bW.numpy(), p.alpha.numpy(), p.x.numpy(), p.num_groups)
     got = run_rowwise(gpu_device, p.bW, p.alpha, p.x, p.num_groups)
-    _assert_close(got, want, (N, K, nb, gs, M))
+    _assert_close(got, want, (N, K, nb, gs, M), margin=_rows_margin(K, gs, M))
+
+
+def _rows_margin(K, gs, M):
+    """Two or more rows through the look-up kernel (shapes the matrix-core kernel does not take: K
+    not a multiple of 128, groups not a multiple of 128 inputs) share one table set whose entries
+    hold two rows as fp16 halves: one more fp16 rounding per table entry, about 3e-4 on the
+    output.  Held to a quarter of the bars instead of a tenth."""
+    on_matrix_cores = M >= 3 and K % 128 == 0 and gs % 128 == 0
+    return TIGHT if M == 1 or on_matrix_cores else PAIR_TABLES
+
+
+@pytest.mark.parametrize("N,K,nb,gs,M", [
+    (512, 288, 3, 32, 2),        # look-up kernel, one pair of rows
+    (512, 288, 4, 96, 3),        # two pairs, the fourth row a repeat of the third
+    (300, 1056, 2, 32, 4),       # two pairs, K tail, N tail
+    (11008, 4096, 3, 128, 2),    # two rows on a sign stream long enough for the look-up kernel
+])
+def test_rows_sharing_pair_tables(gpu_device, N, K, nb, gs, M):
+    p = workload.make_rowwise_problem(N, K, nb=nb, group_size=gs, M=M, seed=N + M, quantize=False)
+    want, _ = orc.gemv_rowwise_c(p.bW.numpy(), p.alpha.numpy(), p.x.numpy(), p.num_groups)
+    got = run_rowwise(gpu_device, p.bW, p.alpha, p.x, p.num_groups)
+    _assert_close(got, want, (N, K, nb, gs, M), margin=PAIR_TABLES)
+    # the rows of a pair do not leak into each other: row 0 alone gives row 0 of the batch to
+    # within the same bar (the single-row kernel uses fp32 tables)
+    one = run_rowwise(gpu_device, p.bW, p.alpha, p.x[:1].contiguous(), p.num_groups)
+    _assert_close(got[:1], one.cpu().numpy(), ("row 0 alone", N, K, nb, gs, M), margin=PAIR_TABLES)
 
 
 def test_rowwise_general_alpha_values(gpu_device):
@@ -272,7 +299,7 @@ def test_uniform_mode(gpu_device, N, K, nb, gs, M):
     _check(native.cabi().lutgemm_gemv_uniform_f16(_ptr(d[0]), _ptr(d[1]), _ptr(d[2]), _ptr(d[3]), _ptr(d_out),
                                                   N, K, nb, K // gs, M, _stream()))
     torch.cuda.synchronize()
-    _assert_close(d_out, want)
+    _assert_close(d_out, want, margin=TIGHT if M == 1 else PAIR_TABLES)   # (uniform mode has no matrix-core path)
 
 
 # ---- the Python operator surface ----------------------------------------------
