@@ -459,8 +459,8 @@ def main():
     configs = None
     if not (args.no_configs or args.plain_only):
         configs = {"note": "us per call = device time of a HIP-graph replay of >= 24 calls over distinct weight sets "
-                           "(> 256 MB in rotation), median of 3; 1 row (and 2 rows above 32 MB of signs) = table look-up "
-                           "kernel, otherwise matrix-core kernel; " + DATA_NOTE}
+                           "(> 256 MB in rotation), median of 3; 1 row (and 2 rows above 12 MB of signs, through fp16-pair "
+                           "tables) = table look-up kernel, otherwise matrix-core kernel; " + DATA_NOTE}
 
         def row_entry(N, K, nb, M, with_oracle):
             cnt = max(3, min(24, (400 << 20) // (K // 8 * N * nb)))
@@ -550,12 +550,12 @@ def main():
             c3[f"{N}x{K}x{nb}bit_R{R}"] = row
         configs["config3_llama13b_block_alpha"] = c3
 
-        # config 5: Llama-2-70B shapes, 2 and 4 bits, 1 / 4 / 16 / 32 rows
+        # config 5: Llama-2-70B shapes, 2 and 4 bits, 1 / 2 / 4 / 16 / 32 rows
         c5 = {}
         for (N, K) in workload.LLAMA2_70B_SHAPES:
             for nb in (2, 4):
                 row = {}
-                for M in (1, 4, 16, 32):
+                for M in (1, 2, 4, 16, 32):
                     # the scalar oracle is affordable up to about a second of look-ups
                     with_oracle = (K // 8) * N * nb * M <= (1 << 30)
                     e, g5 = row_entry(N, K, nb, M, with_oracle)
