@@ -138,10 +138,15 @@ int env_int(const char *name, int fallback)
 // Measured, one row, 256 vs 512 workgroups: 11008x4096x3 8.78 vs 9.04 us, 4096x11008x3 8.59
 // vs 9.12, 13824x5120x2 8.92 vs 9.64, 8192x8192x2 8.27 vs 8.49; 8192x8192x4 11.74 vs 11.06,
 // 28672x8192x2 18.75 vs 16.62.
-int target_blocks(long sign_bytes)
+// The block-alpha formats pay more per item (their alphas are staged per item), so a long
+// range hurts them sooner: beyond four items per workgroup they take two workgroups per CU
+// (13824x5120x2 in eight row groups 9.16 vs 8.58 us, 5120x13824x2 10.0 vs 8.54; 5120x5120x2,
+// 1.6 items per workgroup, 5.91 vs 6.37).
+int target_blocks(long sign_bytes, long items = 0, bool block_alpha = false)
 {
     static const int v = env_int("LUTGEMM_TARGET_BLOCKS", 0);
     if (v > 0) return v;
+    if (block_alpha && items > 4 * 256) return 512;
     return sign_bytes <= (24l << 20) ? 256 : 512;  // 1 or 2 workgroups x 256 CUs
 }
 
@@ -408,7 +413,8 @@ int run(int mode, const uint32_t *bW, const void *alpha, const void *qbias, cons
     if (rc != LUTGEMM_OK) return rc;
     if (mfma_eligible(p, mode)) return run_mfma(p, acc);
     const int mrows = pick_mrows(M);
-    rc = plan_lookup(p, mrows, target_blocks((long)N * (K / 8) * nb));
+    const long items = (long)((N + kTileCols - 1) / kTileCols) * p.nsets;
+    rc = plan_lookup(p, mrows, target_blocks((long)N * (K / 8) * nb, items, mode != kRowF16 && mode != kUniformF16));
     if (rc != LUTGEMM_OK) return rc;
     if (lookup_splits_k(p)) {
         rc = accum_words(acc, (size_t)M * N, &p.accum);
