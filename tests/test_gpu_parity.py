@@ -212,6 +212,9 @@ def test_config5_small_batches(gpu_device, M):
     (272, 384, 3, 128, 33),      # three row chunks, ragged N
     (4096, 4096, 3, 256, 8),     # group of 256 inputs (two K-steps per alpha)
     (11008, 4096, 2, 4096, 32),  # one group along K
+    (22016, 4096, 3, 128, 4),    # 344 tiles: two K-slices each, more workgroups than are resident at once
+    (5120, 13824, 3, 128, 4),    # 108 K-steps in three slices of unequal length
+    (5120, 5120, 3, 128, 16),    # 40 K-steps, slices of 16, 16 and 8
 ])
 def test_small_batch_matrix_core_path(gpu_device, N, K, nb, gs, M):
     p = workload.make_rowwise_problem(N, K, nb=nb, group_size=gs, M=M, seed=N + M, quantize=False)
