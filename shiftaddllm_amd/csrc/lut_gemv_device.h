@@ -887,7 +887,7 @@ __device__ __forceinline__ void gemv_range(const Problem &p, int range, int mchu
     } else {
         // Several rows per pass, per-lane block alphas (the register budget does not allow the
         // first item a code path of its own: up to 300 bytes of spills per lane measured), and
-        // grouped launches.  Everything is requested up front and the first iteration skips its
+        // four-plane problems of grouped launches.  Everything is requested up front and the first iteration skips its
         // first step at run time (opaque, which keeps the compiler from peeling it).
 #pragma clang loop unroll(disable)
         for (int j = 0; j < pairs; ++j) {
@@ -931,9 +931,11 @@ lut_gemv_kernel(const Problem p)
 // Several row-wise problems in one launch.  Bit widths may differ between the
 // problems of a group.
 // XF: the input transform shared by all problems of the launch.
-// (Grouped launches keep the loop that requests two items up front: their ranges hold three
-// or four items, and requesting the second one late costs more than the first one gains:
-// q,k,v + o + gate,up + down of a 7B block 5.06 us per GEMV this way, 5.37 the other.)
+// (Up to three bit planes take the first item on its own, like a lone problem; four planes
+// keep the loop that requests two items up front: with the peeled first item as well the
+// kernel, whose register count is that of its largest bit width, spills 10-19 registers per
+// lane, and everything slows down: q,k,v of a 7B block 10.3 us per launch with the spills,
+// 9.6 with the old loop throughout, 9.1 this way; gate,up 14.4 / 13.4 / 12.8.)
 template <int XF>
 __global__ void __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4, 4)))
 lut_gemv_group_kernel(const Group g)
@@ -948,9 +950,9 @@ lut_gemv_group_kernel(const Group g)
     int range, m;
     decode_block(p, (int)blockIdx.x, range, m);
     switch (p.nb) {
-    case 1: gemv_range<1, kRowF16, 1, XF, true, false>(p, range, m, lut); break;
-    case 2: gemv_range<2, kRowF16, 1, XF, true, false>(p, range, m, lut); break;
-    case 3: gemv_range<3, kRowF16, 1, XF, true, false>(p, range, m, lut); break;
+    case 1: gemv_range<1, kRowF16, 1, XF, true, true>(p, range, m, lut); break;
+    case 2: gemv_range<2, kRowF16, 1, XF, true, true>(p, range, m, lut); break;
+    case 3: gemv_range<3, kRowF16, 1, XF, true, true>(p, range, m, lut); break;
     default: gemv_range<4, kRowF16, 1, XF, true, false>(p, range, m, lut); break;
     }
 }
