@@ -203,6 +203,43 @@ size_t lutgemm_workspace_words(int N, int M);
 int lutgemm_reserve_workspace(void *stream, size_t words);
 
 /*
+ * How a lone call with these sizes would be launched: which kernel, how many
+ * workgroups, how the work is cut.  Pure host arithmetic: no device is touched,
+ * so launch plans can be inspected (and tested) on a machine without a GPU.
+ * `format` is one of LUTGEMM_FORMAT_*; `groups` is num_groups for the row-wise
+ * and uniform formats and the number of row groups R for the block formats.
+ * Returns what the compute entry point would return for the same sizes
+ * (LUTGEMM_EINVAL, LUTGEMM_EUNSUP) without launching anything.  The tuning knobs
+ * of the environment apply as they do to the compute calls.  No counterpart in
+ * the reference, whose launch geometry is fixed at compile time
+ * (mv_fp16_bias.hpp:726-774).
+ */
+#define LUTGEMM_FORMAT_ROWWISE_F16 0
+#define LUTGEMM_FORMAT_BLOCK_F16 1
+#define LUTGEMM_FORMAT_BLOCK_SHIFT_U16 2
+#define LUTGEMM_FORMAT_BLOCK_APOT_I8 3
+#define LUTGEMM_FORMAT_UNIFORM_F16 4
+
+typedef struct lutgemm_plan {
+    int kernel;          /* 0: table look-up kernel, 1: matrix-core kernel */
+    int workgroups;      /* of the launch */
+    int rows_per_pass;   /* activation rows a workgroup handles together */
+    int row_chunks;      /* ceil(M / rows_per_pass) */
+    int tiles;           /* output tiles: 256 columns (look-up), 64 (matrix cores) */
+    int k_units;         /* sets of 256 inputs (look-up), steps of 128 (matrix cores) */
+    /* look-up kernel: the tiles x k_units items of a row chunk, tile-major, are cut into
+     * `ranges` contiguous ranges: the first `long_ranges` of `items_per_long_range`
+     * items, the others of `items_per_short_range` (the last one may be shorter) */
+    int ranges, long_ranges, items_per_long_range, items_per_short_range;
+    /* matrix-core kernel: every tile is cut into `k_slices` slices of
+     * `units_per_slice` steps (the last one may be shorter) */
+    int k_slices, units_per_slice;
+    int needs_workspace; /* 1: the launch uses lutgemm_workspace_words(N, M) accumulator words */
+} lutgemm_plan;
+
+int lutgemm_describe_plan(int format, int N, int K, int nb, int groups, int M, lutgemm_plan *plan);
+
+/*
  * Measurement helpers for the floors any kernel of this library sits on (no
  * counterpart in the reference): a kernel that streams `bytes` (multiple of 16)
  * from `src` with the same 128-bit non-temporal loads as the look-up kernel and

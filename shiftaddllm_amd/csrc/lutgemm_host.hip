@@ -405,23 +405,44 @@ int run_mfma_group(Group &g, const Accum &acc)
     return e == hipSuccess ? LUTGEMM_OK : hip_fail(e);
 }
 
+// Which kernel a lone problem runs on and how it is cut up (no device work).
+enum Kernel : int { kLookup = 0, kMatrixCore = 1 };
+
+int plan_single(Problem &p, int mode, int *kernel, int *mrows)
+{
+    if (mfma_eligible(p, mode)) {
+        const int mt = p.M > 16 ? 2 : 1;
+        Group one{};
+        one.count = 1;
+        one.p[0] = p;
+        plan_mfma(p, mt, mfma_slices(one, mt));
+        *kernel = kMatrixCore;
+        *mrows = 16 * mt;
+        return LUTGEMM_OK;
+    }
+    *kernel = kLookup;
+    *mrows = pick_mrows(p.M);
+    const long items = (long)((p.N + kTileCols - 1) / kTileCols) * p.nsets;
+    return plan_lookup(p, *mrows, target_blocks((long)p.N * (p.K / 8) * p.nb, items, mode != kRowF16 && mode != kUniformF16));
+}
+
 int run(int mode, const uint32_t *bW, const void *alpha, const void *qbias, const void *x,
         void *out, int N, int K, int nb, int num_groups, int M, const Accum &acc)
 {
     Problem p;
     int rc = fill_problem(p, mode, bW, alpha, qbias, x, out, N, K, nb, num_groups, M);
     if (rc != LUTGEMM_OK) return rc;
-    if (mfma_eligible(p, mode)) return run_mfma(p, acc);
-    const int mrows = pick_mrows(M);
-    const long items = (long)((N + kTileCols - 1) / kTileCols) * p.nsets;
-    rc = plan_lookup(p, mrows, target_blocks((long)N * (K / 8) * nb, items, mode != kRowF16 && mode != kUniformF16));
+    int kernel = kLookup, mrows = 1;
+    rc = plan_single(p, mode, &kernel, &mrows);
     if (rc != LUTGEMM_OK) return rc;
-    if (lookup_splits_k(p)) {
+    if (kernel == kMatrixCore ? p.ksplit > 1 : lookup_splits_k(p)) {
         rc = accum_words(acc, (size_t)M * N, &p.accum);
         if (rc != LUTGEMM_OK) return rc;
     }
     hipError_t e;
-    if (mode == kRowF16 || mode == kUniformF16)
+    if (kernel == kMatrixCore)
+        e = launch_mfma(p, mrows / 16, acc.stream);
+    else if (mode == kRowF16 || mode == kUniformF16)
         e = launch_gemv_rowwise(p, mode, mrows, acc.stream);
     else if (p.rows_per_group >= kTileCols)  // a tile spans at most two row groups
         e = launch_gemv_block_staged(p, mode + 4, mrows, acc.stream);
@@ -685,6 +706,40 @@ size_t lutgemm_algorithmic_bytes(int N, int K, int nb, int M, size_t alpha_entri
     const size_t xin = 2u * (size_t)M * (size_t)K;
     const size_t yio = 2u * 2u * (size_t)M * (size_t)N;  // read (accumulate) + write
     return signs + alphas + xin + yio;
+}
+
+int lutgemm_describe_plan(int format, int N, int K, int nb, int groups, int M, lutgemm_plan *plan)
+{
+    if (!plan || format < LUTGEMM_FORMAT_ROWWISE_F16 || format > LUTGEMM_FORMAT_UNIFORM_F16) return LUTGEMM_EINVAL;
+    // (nothing is dereferenced while planning: any aligned non-null address will do)
+    static const uint64_t dummy[2] = {0, 0};
+    Problem p;
+    int rc = fill_problem(p, format, (const uint32_t *)dummy, dummy, dummy, dummy, (void *)dummy, N, K, nb, groups, M);
+    if (rc != LUTGEMM_OK) return rc;
+    int kernel = kLookup, mrows = 1;
+    rc = plan_single(p, format, &kernel, &mrows);
+    if (rc != LUTGEMM_OK) return rc;
+    *plan = lutgemm_plan{};
+    plan->kernel = kernel;
+    plan->workgroups = p.n_blocks;
+    plan->rows_per_pass = mrows;
+    plan->row_chunks = p.mchunks;
+    if (kernel == kMatrixCore) {
+        plan->tiles = p.n_tiles;
+        plan->k_units = p.nsets;
+        plan->k_slices = p.ksplit;
+        plan->units_per_slice = p.sets_per_split;
+        plan->needs_workspace = p.ksplit > 1;
+    } else {
+        plan->tiles = p.n_tiles;
+        plan->k_units = p.nsets;
+        plan->long_ranges = p.long_ranges;
+        plan->items_per_long_range = p.items_per_wg;
+        plan->items_per_short_range = p.short_items;
+        plan->ranges = p.wgs_per_chunk;
+        plan->needs_workspace = lookup_splits_k(p);
+    }
+    return LUTGEMM_OK;
 }
 
 size_t lutgemm_workspace_words(int N, int M)

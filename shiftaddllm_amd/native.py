@@ -32,6 +32,7 @@ C_ABI_SYMBOLS = (
     "lutgemm_copy_bytes",
     "lutgemm_workspace_words",
     "lutgemm_reserve_workspace",
+    "lutgemm_describe_plan",
     "lutgemm_measure_stream_read",
     "lutgemm_measure_empty_launch",
     "lutgemm_release_workspaces",
@@ -50,6 +51,13 @@ class RowwiseProblem(ctypes.Structure):
     _fields_ = [("bW", ctypes.c_void_p), ("alpha_f16", ctypes.c_void_p), ("x_f16", ctypes.c_void_p),
                 ("out_f16", ctypes.c_void_p), ("N", ctypes.c_int), ("K", ctypes.c_int),
                 ("nb", ctypes.c_int), ("num_groups", ctypes.c_int), ("M", ctypes.c_int)]
+
+
+class Plan(ctypes.Structure):
+    """struct lutgemm_plan of include/lutgemm_gfx950.h."""
+    _fields_ = [(n, ctypes.c_int) for n in (
+        "kernel", "workgroups", "rows_per_pass", "row_chunks", "tiles", "k_units", "ranges", "long_ranges",
+        "items_per_long_range", "items_per_short_range", "k_slices", "units_per_slice", "needs_workspace")]
 
 
 class FusedProblem(ctypes.Structure):
@@ -122,6 +130,8 @@ def cabi() -> ctypes.CDLL:
         lib.lutgemm_algorithmic_bytes.restype = sz
         lib.lutgemm_copy_bytes.argtypes = [vp, vp, sz, vp]
         lib.lutgemm_copy_bytes.restype = ci
+        lib.lutgemm_describe_plan.argtypes = [ci, ci, ci, ci, ci, ci, ctypes.POINTER(Plan)]
+        lib.lutgemm_describe_plan.restype = ci
         lib.lutgemm_workspace_words.argtypes = [ci, ci]
         lib.lutgemm_workspace_words.restype = sz
         lib.lutgemm_reserve_workspace.argtypes = [vp, sz]

@@ -1,0 +1,140 @@
+"""Launch plans without a GPU: lutgemm_describe_plan is pure host arithmetic, so the
+planner's invariants are checked here over the benchmark shapes and a few thousand
+random ones.  What a kernel relies on (and cannot check itself):
+  look-up kernel   the ranges cover every (tile, set) item exactly once, none is empty,
+                   and no output tile receives more than 32 contributions (the count field
+                   of an accumulator word, lutgemm_common.h);
+  matrix cores     the K-slices cover every step, none is empty, each is a whole number of
+                   eight-step rounds, and there are at most 32 of them per tile."""
+import ctypes
+import os
+import random
+
+import pytest
+
+LOOKUP, MATRIX_CORE = 0, 1
+ROWWISE, BLOCK_F16, BLOCK_U16, BLOCK_I8, UNIFORM = range(5)
+MAX_CONTRIB = 32
+
+
+@pytest.fixture(scope="module")
+def lib():
+    from shiftaddllm_amd import native
+    if not os.path.exists(native.KERNEL_LIB):
+        from shiftaddllm_amd import build
+        build.build_kernel_library()
+    return native.cabi()
+
+
+def describe(lib, fmt, N, K, nb, groups, M):
+    from shiftaddllm_amd import native
+    plan = native.Plan()
+    rc = lib.lutgemm_describe_plan(fmt, N, K, nb, groups, M, ctypes.byref(plan))
+    return rc, plan
+
+
+def check_plan(p, N, K, M):
+    assert p.workgroups >= 1 and p.row_chunks == -(-M // p.rows_per_pass)
+    if p.kernel == LOOKUP:
+        assert p.tiles == -(-N // 256) and p.k_units == -(-K // 256)
+        total = p.tiles * p.k_units
+        a, b, n_long, n = p.items_per_long_range, p.items_per_short_range, p.long_ranges, p.ranges
+        assert a >= b >= 1 and 1 <= n_long <= n and p.workgroups == n * p.row_chunks
+        starts = [min(r, n_long) * a + max(r - n_long, 0) * b for r in range(n + 1)]
+        assert starts[n] >= total, "ranges must cover every item"
+        assert starts[n - 1] < total, "no range may be empty"
+        # contributions per tile = ranges overlapping its k_units items
+        bounds = starts[:n] + [total]
+        worst, split = 0, False
+        r = 0
+        for t in range(p.tiles):
+            lo, hi = t * p.k_units, (t + 1) * p.k_units
+            while bounds[r + 1] <= lo:
+                r += 1
+            c, rr = 1, r
+            while bounds[rr + 1] < hi:
+                rr += 1
+                c += 1
+            worst = max(worst, c)
+            split = split or c > 1
+        assert worst <= MAX_CONTRIB, worst
+        assert bool(p.needs_workspace) >= split, "a tile shared between ranges needs accumulator words"
+    else:
+        assert p.tiles == -(-N // 64) and p.k_units == K // 128
+        assert p.rows_per_pass in (16, 32)
+        assert 1 <= p.k_slices <= MAX_CONTRIB and p.units_per_slice % 8 == 0
+        assert p.k_slices * p.units_per_slice >= p.k_units, "slices must cover every K-step"
+        assert (p.k_slices - 1) * p.units_per_slice < p.k_units, "no slice may be empty"
+        assert p.workgroups == p.tiles * p.k_slices * p.row_chunks
+        assert bool(p.needs_workspace) == (p.k_slices > 1)
+
+
+BENCH_SHAPES = [(3072, 768), (4096, 4096), (11008, 4096), (4096, 11008), (5120, 5120), (13824, 5120), (5120, 13824),
+                (8192, 8192), (28672, 8192), (8192, 28672), (1024, 8192), (22016, 4096), (32000, 4096)]
+
+
+@pytest.mark.parametrize("N,K", BENCH_SHAPES)
+def test_benchmark_shapes_every_bit_width_and_batch(lib, N, K):
+    for nb in (1, 2, 3, 4):
+        for M in (1, 2, 3, 4, 8, 16, 17, 32, 33, 64):
+            rc, p = describe(lib, ROWWISE, N, K, nb, K // 128, M)
+            assert rc == 0, (N, K, nb, M, rc)
+            check_plan(p, N, K, M)
+        for fmt in (BLOCK_F16, BLOCK_U16, BLOCK_I8):
+            for M in (1, 2, 5):
+                rc, p = describe(lib, fmt, N, K, nb, 8, M)
+                assert rc == 0 and p.kernel == LOOKUP
+                check_plan(p, N, K, M)
+
+
+def test_which_kernel_takes_what(lib):
+    # one row: always the look-up kernel; three rows and more of an eligible problem: matrix cores
+    assert describe(lib, ROWWISE, 4096, 4096, 3, 32, 1)[1].kernel == LOOKUP
+    assert describe(lib, ROWWISE, 4096, 4096, 3, 32, 3)[1].kernel == MATRIX_CORE
+    assert describe(lib, ROWWISE, 4096, 4096, 3, 32, 32)[1].rows_per_pass == 32
+    # two rows: matrix cores on short sign streams, the look-up kernel (both rows per pass) on long ones
+    assert describe(lib, ROWWISE, 4096, 4096, 3, 32, 2)[1].kernel == MATRIX_CORE
+    big = describe(lib, ROWWISE, 28672, 8192, 4, 64, 2)[1]
+    assert big.kernel == LOOKUP and big.rows_per_pass == 2 and big.row_chunks == 1
+    # not eligible for the matrix cores: K not a multiple of 128, groups of 32 inputs, other formats
+    assert describe(lib, ROWWISE, 1024, 288, 3, 9, 8)[1].kernel == LOOKUP
+    assert describe(lib, ROWWISE, 1024, 1024, 3, 32, 8)[1].kernel == LOOKUP
+    assert describe(lib, UNIFORM, 1024, 1024, 3, 8, 8)[1].kernel == LOOKUP
+    # the 70B shapes at one row run two workgroups per CU with unequal ranges
+    p = describe(lib, ROWWISE, 28672, 8192, 4, 64, 1)[1]
+    assert p.ranges == 512 and p.long_ranges == 256 and p.items_per_long_range > p.items_per_short_range
+    # the 7B gate|up pair as one problem at eight rows: two K-slices per tile (more workgroups than are resident)
+    assert describe(lib, ROWWISE, 22016, 4096, 3, 32, 8)[1].k_slices == 2
+
+
+def test_random_shapes(lib):
+    rng = random.Random(1234)
+    seen = {LOOKUP: 0, MATRIX_CORE: 0}
+    for i in range(4000):
+        if i % 2:                                    # shapes the matrix-core kernel takes at three rows and more
+            K = 128 * rng.randint(1, 300)
+            N = 16 * rng.randint(1, 2250)
+        else:
+            K = 32 * rng.randint(1, 1200)
+            N = 4 * rng.randint(1, 9000)
+        nb = rng.randint(1, 4)
+        M = rng.choice((1, 1, 1, 2, 3, 4, 7, 16, 17, 40, 100))
+        divisors = [g for g in ((128, 256, 512, K) if i % 2 else (32, 64, 96, 128, 256, 512, K)) if K % g == 0]
+        gs = rng.choice(divisors)
+        rc, p = describe(lib, ROWWISE, N, K, nb, K // gs, M)
+        if rc != 0:
+            assert rc == -3, (N, K, nb, gs, M, rc)      # LUTGEMM_EUNSUP: beyond the exact-division bounds
+            continue
+        check_plan(p, N, K, M)
+        seen[p.kernel] += 1
+    assert seen[LOOKUP] > 500 and seen[MATRIX_CORE] > 100
+
+
+def test_bad_arguments(lib):
+    from shiftaddllm_amd import native
+    plan = native.Plan()
+    assert lib.lutgemm_describe_plan(ROWWISE, 4096, 4096, 3, 32, 1, None) == -1
+    assert lib.lutgemm_describe_plan(9, 4096, 4096, 3, 32, 1, ctypes.byref(plan)) == -1
+    assert lib.lutgemm_describe_plan(ROWWISE, 4096, 4100, 3, 32, 1, ctypes.byref(plan)) == -1   # K % 32
+    assert lib.lutgemm_describe_plan(ROWWISE, 4096, 4096, 5, 32, 1, ctypes.byref(plan)) == -1   # bit planes
+    assert lib.lutgemm_describe_plan(ROWWISE, 4096, 4096, 3, 32, 0, ctypes.byref(plan)) == -1   # rows
