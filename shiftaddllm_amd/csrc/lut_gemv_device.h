@@ -887,8 +887,9 @@ __device__ __forceinline__ void gemv_range(const Problem &p, int range, int mchu
     } else {
         // Several rows per pass, per-lane block alphas (the register budget does not allow the
         // first item a code path of its own: up to 300 bytes of spills per lane measured), and
-        // four-plane problems of grouped launches.  Everything is requested up front and the first iteration skips its
-        // first step at run time (opaque, which keeps the compiler from peeling it).
+        // four-plane problems of grouped launches.  Everything is requested up front and the
+        // first iteration skips its first step at run time (opaque, which keeps the compiler
+        // from peeling it).
 #pragma clang loop unroll(disable)
         for (int j = 0; j < pairs; ++j) {
             int first = __builtin_amdgcn_readfirstlane(j == 0);
