@@ -372,16 +372,39 @@ __device__ __forceinline__ void lookup_item(const ItemOperands<NB, MODE> &cur, c
             for (int j = 0; j < 4; ++j) av[j] = a4[(j + q) & 3];
         }
     };
+    // Row-wise alphas: the entries of a bit plane are summed as they are and the plane's
+    // alpha is applied once, after the item's last look-up, so the alphas (requested after
+    // the sign words) are not waited for before that.
+    [[maybe_unused]] float part[NB][4];
+    if constexpr (MODE == kRowF16) {
+#pragma unroll
+        for (int b = 0; b < NB; ++b)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) part[b][i] = 0.0f;
+    }
     auto retire = [&](int u, const float (&v)[8], const float (&av)[4]) {
         const int b = u >> 1, i0 = (u & 1) * 2;
-        [[maybe_unused]] const uint32_t ar = (u & 1) ? cur.a_row[b].y : cur.a_row[b].x;
+        if constexpr (MODE == kRowF16) {
+#pragma unroll
+            for (int i = 0; i < 2; ++i)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) part[b][i0 + i] += v[4 * i + j];
+            if (u == kUnits - 1) {
+#pragma unroll
+                for (int bb = 0; bb < NB; ++bb) {
+                    const uint32_t a2[2] = {cur.a_row[bb].x, cur.a_row[bb].y};
+#pragma unroll
+                    for (int i = 0; i < 4; ++i)
+                        acc[i] = fmaf(part[bb][i], half_bits_to_float((a2[i >> 1] >> (16 * (i & 1))) & 0xffffu), acc[i]);
+                }
+            }
+            return;
+        }
         [[maybe_unused]] const uint32_t au = (u & 1) ? cur.a_uni.y : cur.a_uni.x;
 #pragma unroll
         for (int i = 0; i < 2; ++i) {
             float a = 0.0f;
-            if constexpr (MODE == kRowF16)
-                a = half_bits_to_float((ar >> (16 * i)) & 0xffffu);
-            else if constexpr (MODE == kUniformF16)
+            if constexpr (MODE == kUniformF16)
                 a = half_bits_to_float((au >> (16 * i)) & 0xffffu) * (1.0f / (float)(2 << b));
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
