@@ -712,7 +712,7 @@ int lutgemm_describe_plan(int format, int N, int K, int nb, int groups, int M, l
 {
     if (!plan || format < LUTGEMM_FORMAT_ROWWISE_F16 || format > LUTGEMM_FORMAT_UNIFORM_F16) return LUTGEMM_EINVAL;
     // (nothing is dereferenced while planning: any aligned non-null address will do)
-    static const uint64_t dummy[2] = {0, 0};
+    alignas(16) static const uint64_t dummy[2] = {0, 0};
     Problem p;
     int rc = fill_problem(p, format, (const uint32_t *)dummy, dummy, dummy, dummy, (void *)dummy, N, K, nb, groups, M);
     if (rc != LUTGEMM_OK) return rc;
