@@ -3,24 +3,37 @@
 // The problem is the kernel argument itself and the bit width a template parameter, so
 // that the start of the kernel is the plain kernel's: one round of scalar loads, no
 // dispatch on the problem's fields.
+#include <stdlib.h>
+
 #include "lut_gemv_device.h"
 #include "lutgemm_launch.h"
 
 namespace lutgemm {
 namespace {
 
-template <int NB, int XF>
+// SINGLE: every range of the launch holds exactly one item.
+template <int NB, int XF, bool SINGLE = false>
 __global__ void __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4, 4)))
 lut_gemv_fused_kernel(const Problem p)
 {
     __shared__ __attribute__((aligned(16))) float lut[kLutDwords + kStageDwords + kWindowDwords];
-    gemv_range<NB, kRowF16, 1, XF, true>(p, (int)blockIdx.x, (int)blockIdx.y, lut);  // grid = (ranges, rows)
+    gemv_range<NB, kRowF16, 1, XF, true, SINGLE ? 2 : 1>(p, (int)blockIdx.x, (int)blockIdx.y, lut);  // grid = (ranges, rows)
 }
 
 template <int NB>
 hipError_t launch_nb(const Problem &p, int xform, hipStream_t stream)
 {
     const dim3 grid((unsigned)p.wgs_per_chunk, (unsigned)p.mchunks), block(kThreads);
+    static const bool single_item = !(getenv("LUTGEMM_SINGLE_ITEM") && *getenv("LUTGEMM_SINGLE_ITEM") == '0');
+    if (p.items_per_wg == 1 && p.short_items == 1 && single_item) {
+        if (xform == kXNorm)
+            hipLaunchKernelGGL((lut_gemv_fused_kernel<NB, kXNorm, true>), grid, block, 0, stream, p);
+        else if (xform == kXGate)
+            hipLaunchKernelGGL((lut_gemv_fused_kernel<NB, kXGate, true>), grid, block, 0, stream, p);
+        else
+            hipLaunchKernelGGL((lut_gemv_fused_kernel<NB, kXNone, true>), grid, block, 0, stream, p);
+        return hipGetLastError();
+    }
     if (xform == kXNorm)
         hipLaunchKernelGGL((lut_gemv_fused_kernel<NB, kXNorm>), grid, block, 0, stream, p);
     else if (xform == kXGate)

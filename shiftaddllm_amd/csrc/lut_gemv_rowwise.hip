@@ -20,6 +20,7 @@ template <int NB, int MODE>
 hipError_t launch_nb(const Problem &p, int mrows, hipStream_t stream)
 {
     static const bool pair_tables = pair_tables_enabled();
+    static const bool single_item = !(getenv("LUTGEMM_SINGLE_ITEM") && *getenv("LUTGEMM_SINGLE_ITEM") == '0');
     const dim3 grid((unsigned)p.wgs_per_chunk, (unsigned)p.mchunks), block(kThreads);
     if (mrows == 4 && pair_tables)
         hipLaunchKernelGGL((lut_gemv_kernel<NB, MODE, 4, true>), grid, block, 0, stream, p);
@@ -29,6 +30,8 @@ hipError_t launch_nb(const Problem &p, int mrows, hipStream_t stream)
         hipLaunchKernelGGL((lut_gemv_kernel<NB, MODE, 4>), grid, block, 0, stream, p);
     else if (mrows == 2)
         hipLaunchKernelGGL((lut_gemv_kernel<NB, MODE, 2>), grid, block, 0, stream, p);
+    else if (p.items_per_wg == 1 && p.short_items == 1 && single_item)
+        hipLaunchKernelGGL((lut_gemv_kernel<NB, MODE, 1, false, true>), grid, block, 0, stream, p);
     else
         hipLaunchKernelGGL((lut_gemv_kernel<NB, MODE, 1>), grid, block, 0, stream, p);
     return hipGetLastError();
