@@ -640,7 +640,8 @@ def main():
         "dependency_branches": branched,
         "roofline": {"bound": "hbm", "achieved": round(achieved_gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved_gbs / HBM_PEAK_GBS, 4), "traffic": traffic,
-                     "kernel": "lut_gemv_kernel<3, 0, 1> (nb=3, row-wise alpha, 1 row)",
+                     "kernel": "lut_gemv_kernel<3, 0, 1, false, *> (nb=3, row-wise alpha, 1 row; the 4096x4096 launches, "
+                               "one item per workgroup, take the single-item instance)",
                      "algorithmic_bytes_per_launch": round(mean_bytes),
                      "avg_launch_us": round(value_us, 4),
                      "measured": "224 launches one after the other on one stream (graph replay), HIP events on that stream",
