@@ -9,7 +9,9 @@ template <int NB>
 hipError_t launch_nb(const Problem &p, int mt, hipStream_t stream)
 {
     const dim3 grid((unsigned)p.n_blocks), block(kMfmaThreads);
-    if (mt == 2)
+    if (mt == 1 && p.sets_per_split == kMfmaWaves)  // one round per K-slice
+        hipLaunchKernelGGL((lut_gemm_mfma_kernel<NB, 1, true>), grid, block, 0, stream, p);
+    else if (mt == 2)
         hipLaunchKernelGGL((lut_gemm_mfma_kernel<NB, 2>), grid, block, 0, stream, p);
     else
         hipLaunchKernelGGL((lut_gemm_mfma_kernel<NB, 1>), grid, block, 0, stream, p);
@@ -20,7 +22,9 @@ template <int NB>
 hipError_t launch_fused_nb(const Problem &p, int mt, hipStream_t stream)
 {
     const dim3 grid((unsigned)p.n_blocks), block(kMfmaThreads);
-    if (mt == 2)
+    if (mt == 1 && p.sets_per_split == kMfmaWaves)  // one round per K-slice
+        hipLaunchKernelGGL((lut_gemm_mfma_fused_kernel<NB, 1, true>), grid, block, 0, stream, p);
+    else if (mt == 2)
         hipLaunchKernelGGL((lut_gemm_mfma_fused_kernel<NB, 2>), grid, block, 0, stream, p);
     else
         hipLaunchKernelGGL((lut_gemm_mfma_fused_kernel<NB, 1>), grid, block, 0, stream, p);

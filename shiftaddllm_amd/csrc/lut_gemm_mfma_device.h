@@ -101,7 +101,9 @@ __device__ __forceinline__ f16x8 expand_signs(uint32_t w, int beta, uint32_t alp
 // xs: kMfmaLdsBytes<MT> bytes of LDS for the final reduction (and, behind them, the
 // reciprocal RMS of the tile's rows).
 // EXTRA: the launch honours the split-RMSNorm fields of the problem (next_in, sumsq_*).
-template <int NB, int MT, bool EXTRA = false>
+// ONE: every K-slice of the launch is a single round, i.e. a wave takes at most one step (the
+//      host's choice): nothing is requested beyond that step.
+template <int NB, int MT, bool EXTRA = false, bool ONE = false>
 __device__ __forceinline__ void mfma_tile(const Problem &p, int local_block, char *xs)
 {
     const int tid = threadIdx.x;
@@ -217,7 +219,17 @@ __device__ __forceinline__ void mfma_tile(const Problem &p, int local_block, cha
     const int last_step = p.nsets - 1;
     const int first_step = step_begin + wave;
     const int n_steps = first_step < step_end ? (step_end - first_step + kMfmaWaves - 1) / kMfmaWaves : 0;
-    const int pairs = (n_steps + 1) / 2;
+    const int pairs = ONE ? 0 : (n_steps + 1) / 2;
+    if constexpr (ONE) {
+        // One round per slice: the general loop would request a second, discarded step behind
+        // the first one, and a wave cannot end before those loads have come back.
+        mfma_load<NB, MT>(opA, p, min(first_step, last_step), kb, wcol4, xlane);
+        __builtin_amdgcn_sched_barrier(0);
+        if constexpr (EXTRA)
+            if (scaled) row_scales();
+        __builtin_amdgcn_sched_barrier(0);
+        if (n_steps > 0) compute(opA);
+    }
 #pragma clang loop unroll(disable)
     for (int j = 0; j < pairs; ++j) {
         // (opaque, which keeps the compiler from peeling the first iteration)
@@ -234,8 +246,8 @@ __device__ __forceinline__ void mfma_tile(const Problem &p, int local_block, cha
         __builtin_amdgcn_sched_barrier(0);
         compute(opA);
     }
-    if (n_steps > 0 && (n_steps & 1) == 0) compute(opB);
-    if constexpr (EXTRA)
+    if (!ONE && n_steps > 0 && (n_steps & 1) == 0) compute(opB);
+    if constexpr (EXTRA && !ONE)
         if (n_steps == 0 && scaled) row_scales();  // (a wave without steps still owes its rows)
 
     // ---- the 8 waves' accumulators meet in LDS -----------------------------------
@@ -311,19 +323,19 @@ __device__ __forceinline__ void mfma_tile(const Problem &p, int local_block, cha
     }
 }
 
-template <int NB, int MT>
+template <int NB, int MT, bool ONE = false>
 __global__ void __launch_bounds__(kMfmaThreads) lut_gemm_mfma_kernel(const Problem p)
 {
     __shared__ __attribute__((aligned(16))) char xs[kMfmaLdsBytes<MT>];
-    mfma_tile<NB, MT>(p, (int)blockIdx.x, xs);
+    mfma_tile<NB, MT, false, ONE>(p, (int)blockIdx.x, xs);
 }
 
 // One problem with the split-RMSNorm fields honoured.
-template <int NB, int MT>
+template <int NB, int MT, bool ONE = false>
 __global__ void __launch_bounds__(kMfmaThreads) lut_gemm_mfma_fused_kernel(const Problem p)
 {
     __shared__ __attribute__((aligned(16))) char xs[kMfmaLdsBytes<MT>];
-    mfma_tile<NB, MT, true>(p, (int)blockIdx.x, xs);
+    mfma_tile<NB, MT, true, ONE>(p, (int)blockIdx.x, xs);
 }
 
 // Several problems in one launch; bit widths may differ.
