@@ -213,12 +213,14 @@ __device__ __forceinline__ void mfma_tile(const Problem &p, int local_block, cha
     // each step's loads are issued one compute phase ahead.  Steps are taken in pairs by
     // a counted loop with one load site per buffer (a second site makes the register
     // allocator reconcile the two with copies that wait for the loads): the first
-    // iteration skips its first compute at run time, and loads beyond the wave's last
-    // step re-read a clamped address and are discarded, so that the waits can count them.
+    // iteration skips its first compute at run time, and a load beyond the wave's last
+    // step re-reads that last step (the lines the wave has just asked for) and is
+    // discarded, so that the waits can count it.
     MfmaOperands<NB, MT> opA, opB;
     const int last_step = p.nsets - 1;
     const int first_step = step_begin + wave;
     const int n_steps = first_step < step_end ? (step_end - first_step + kMfmaWaves - 1) / kMfmaWaves : 0;
+    const int own_last = n_steps > 0 ? first_step + kMfmaWaves * (n_steps - 1) : last_step;
     const int pairs = ONE ? 0 : (n_steps + 1) / 2;
     if constexpr (ONE) {
         // One round per slice: the general loop would request a second, discarded step behind
@@ -236,13 +238,13 @@ __device__ __forceinline__ void mfma_tile(const Problem &p, int local_block, cha
         int first = __builtin_amdgcn_readfirstlane(j == 0);
         asm volatile("" : "+s"(first));
         const int s = first_step + 2 * kMfmaWaves * j;
-        mfma_load<NB, MT>(opA, p, min(s, last_step), kb, wcol4, xlane);
+        mfma_load<NB, MT>(opA, p, min(s, own_last), kb, wcol4, xlane);
         __builtin_amdgcn_sched_barrier(0);
         if (!first) compute(opB);
         if constexpr (EXTRA)
             if (first && scaled) row_scales();
         __builtin_amdgcn_sched_barrier(0);
-        mfma_load<NB, MT>(opB, p, min(s + kMfmaWaves, last_step), kb, wcol4, xlane);
+        mfma_load<NB, MT>(opB, p, min(s + kMfmaWaves, own_last), kb, wcol4, xlane);
         __builtin_amdgcn_sched_barrier(0);
         compute(opA);
     }
