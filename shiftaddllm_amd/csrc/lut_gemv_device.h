@@ -41,8 +41,7 @@
 //    the sum, adds the caller's fp16 output, rounds once and clears the word.
 //    Integer addition is associative: the result does not depend on arrival
 //    order.  No fences (a device-scope release costs tens of microseconds here)
-//    and no second pass.  In "deferred" mode the atomics do not return and
-//    nobody finishes: a later kernel reads the words.
+//    and no second pass.
 #ifndef LUT_GEMV_DEVICE_H
 #define LUT_GEMV_DEVICE_H
 
@@ -751,17 +750,13 @@ __device__ __forceinline__ void gemv_range(const Problem &p, int range, int mchu
             if (!owner || n >= p.N || m >= p.M) continue;
             __half *dst = p.out + (size_t)m * p.N + n;
             const float prev = p.overwrite ? 0.0f : half_bits_to_float(out_prev[r]);
-            if (count == 1 && p.finish == kFinishInline) {
+            if (count == 1) {
                 complete(r, dst, prev + v);
                 continue;
             }
             unsigned long long *word = p.accum + (size_t)m * p.N + n;
             const Contribution c = fixed_contribution(v);
             if (c.flags) __hip_atomic_fetch_or(word, c.flags, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            if (p.finish == kFinishDefer) {
-                __hip_atomic_fetch_add(word, c.add, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                continue;
-            }
             const unsigned long long old =
                 __hip_atomic_fetch_add(word, c.add, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             if ((int)(old >> 56) != count - 1) continue;

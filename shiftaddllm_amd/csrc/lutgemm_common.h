@@ -65,10 +65,6 @@ constexpr int base_mode(int mode) { return is_staged(mode) ? mode - 4 : mode; }
 // compile-time input transform of a kernel instance
 constexpr int kXNone = 0, kXNorm = 1, kXGate = 2;
 
-// how a workgroup hands over its partial sums (Problem::finish)
-constexpr int kFinishInline = 0;  // returning atomics; the last contributor rounds and writes `out`
-constexpr int kFinishDefer = 1;   // non-returning atomics; a later kernel reads and clears the words
-
 // Division by a run-time constant without a divide: n / d == umulhi((2 * n) >> shift,
 // magic), with the pair prepared on the host (kernels here start and end within a
 // few microseconds; a software division is some thirty instructions on that path).
@@ -148,7 +144,7 @@ struct Problem {
     int sets_per_split;
     int ksplit;
     float norm_eps;
-    int finish;          // kFinishInline / kFinishDefer
+    int reserved_;
     // ---- cache line 3: needed when sums are handed over --------------------------------------
     int overwrite;       // 1: out = y instead of out += y
     // RMSNorm split over two launches (fused entry point only).  The launch that completes

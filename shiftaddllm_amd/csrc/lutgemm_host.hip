@@ -210,7 +210,7 @@ int plan_lookup(Problem &p, int mrows, long want_blocks)
 // true when some tile is shared between ranges, i.e. accumulator words are needed
 bool lookup_splits_k(const Problem &p)
 {
-    if (p.finish == kFinishDefer || p.items_per_wg % p.nsets != 0) return true;
+    if (p.items_per_wg % p.nsets != 0) return true;
     return p.wgs_per_chunk > p.long_ranges && (p.short_items % p.nsets != 0 || p.split_item % p.nsets != 0);
 }
 
