@@ -225,6 +225,48 @@ def test_small_batch_matrix_core_path(gpu_device, N, K, nb, gs, M):
     assert torch.equal(got, run_rowwise(gpu_device, p.bW, p.alpha, p.x, p.num_groups, out=bias))
 
 
+def test_random_shapes_against_a_dense_product(gpu_device):
+    """240 seeded random problems (any K % 32, N % 4, group size, 1-4 bit planes, 1-33 rows, general
+    fp16 alphas, a bias in `out`) against the dense fp64 product of the dequantised matrix, formed on
+    the GPU by framework operations: a reference that shares nothing with the oracle's look-up
+    formulation.  Every launch plan the planner has is hit (checked through lutgemm_describe_plan)."""
+    import random
+    dev = gpu_device
+    lib = native.cabi()
+    rng = random.Random(2024)
+    plan = native.Plan()
+    seen = set()
+    for case in range(240):
+        if case % 3 == 0:     # shapes the matrix-core kernel takes from three rows on
+            K = 128 * rng.randint(1, 64)
+            N = 16 * rng.randint(1, 500)
+            gs = rng.choice([g for g in (128, 256, 512, K) if K % g == 0])
+        else:
+            K = 32 * rng.randint(1, 200)
+            N = 4 * rng.randint(1, 1800)
+            gs = rng.choice([g for g in (32, 64, 96, 128, 256, K) if K % g == 0])
+        nb = rng.randint(1, 4)
+        M = rng.choice((1, 1, 1, 2, 2, 3, 4, 5, 8, 16, 17, 33))
+        g = torch.Generator(device=dev).manual_seed(case)
+        bW = torch.randint(-2 ** 31, 2 ** 31 - 1, (K // 32, nb, N), generator=g, device=dev, dtype=torch.int32)
+        alpha = (torch.rand((K // gs, nb, N), generator=g, device=dev) * 0.02 + 0.001).half()
+        x = torch.randn((M, K), generator=g, device=dev).half()
+        bias = torch.randn((M, N), generator=g, device=dev).half()
+        out = bias.clone()
+        _check(lib.lutgemm_gemv_rowwise_f16(_ptr(bW), _ptr(alpha), _ptr(x), _ptr(out), N, K, nb, K // gs, M, _stream()))
+        torch.cuda.synchronize()
+        signs = ((bW.unsqueeze(1) >> torch.arange(32, device=dev).view(1, 32, 1, 1)) & 1).double() * 2 - 1
+        Wq = (signs.reshape(K, nb, N) * alpha.double().repeat_interleave(gs, dim=0)).sum(1)      # [K][N]
+        want = bias.double() + x.double() @ Wq
+        rel = ((out.double() - want).norm() / want.norm()).item()
+        mad = ((out.double() - want).abs().max() / want.abs().max()).item()
+        _check(lib.lutgemm_describe_plan(0, N, K, nb, K // gs, M, ctypes.byref(plan)))
+        seen.add((plan.kernel, plan.rows_per_pass))
+        # against an un-rounded reference: a quarter of the bars (the final fp16 rounding alone is 2e-4)
+        assert rel <= REL_L2_BAR * 0.25 and mad <= MAX_ABS_BAR * 0.25, (N, K, nb, gs, M, rel, mad)
+    assert seen == {(0, 1), (0, 2), (0, 4), (1, 16), (1, 32)}, seen
+
+
 def test_batch_rows_agree_with_single_row_calls(gpu_device):
     # every row of a batched call equals the batch-1 call on that row (different kernels)
     p = workload.make_rowwise_problem(2048, 2048, nb=3, group_size=128, M=8, seed=77, quantize=False)
