@@ -25,19 +25,34 @@ constexpr int kThreads = 256;
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
-__device__ __forceinline__ float wave_sum(float v)
+// The value of another lane of the same row of 16, by a data-parallel-primitive move.
+template <int CTRL>
+__device__ __forceinline__ float dpp_lane(float v)
 {
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
-    return v;
+    const int vi = __builtin_bit_cast(int, v);
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(vi, vi, CTRL, 0xf, 0xf, false));
 }
 
-__device__ __forceinline__ float wave_max(float v)
+// Sum / maximum over the 64 lanes of a wave on the vector ALU: xor 1 and 2 inside quads, the
+// mirrored quad and the mirrored half of each row of 16, then the four rows by lane reads.
+template <bool MAX>
+__device__ __forceinline__ float wave_reduce(float v)
 {
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, 64));
-    return v;
+    auto op = [](float a, float b) { return MAX ? fmaxf(a, b) : a + b; };
+    v = op(v, dpp_lane<0xb1>(v));   // quad_perm [1,0,3,2]
+    v = op(v, dpp_lane<0x4e>(v));   // quad_perm [2,3,0,1]
+    v = op(v, dpp_lane<0x141>(v));  // row_half_mirror
+    v = op(v, dpp_lane<0x140>(v));  // row_mirror
+    const int vi = __builtin_bit_cast(int, v);
+    const float r0 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(vi, 0));
+    const float r1 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(vi, 16));
+    const float r2 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(vi, 32));
+    const float r3 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(vi, 48));
+    return op(op(r0, r1), op(r2, r3));
 }
+
+__device__ __forceinline__ float wave_sum(float v) { return wave_reduce<false>(v); }
+__device__ __forceinline__ float wave_max(float v) { return wave_reduce<true>(v); }
 
 // Sum (or max) over the 256 threads of a workgroup; `red` holds 4 floats.
 template <bool MAX>
@@ -49,14 +64,6 @@ __device__ __forceinline__ float block_reduce(float v, float *red)
     __syncthreads();
     const float a = red[0], b = red[1], c = red[2], d = red[3];
     return MAX ? fmaxf(fmaxf(a, b), fmaxf(c, d)) : (a + b) + (c + d);
-}
-
-// The value of another lane of the same row of 16, by a data-parallel-primitive move.
-template <int CTRL>
-__device__ __forceinline__ float dpp_lane(float v)
-{
-    const int vi = __builtin_bit_cast(int, v);
-    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(vi, vi, CTRL, 0xf, 0xf, false));
 }
 
 __device__ __forceinline__ void unpack8(const u32x4 &v, float f[8])
