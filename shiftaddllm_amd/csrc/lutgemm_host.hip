@@ -520,19 +520,47 @@ int run_group(int count, const lutgemm_fused_problem *problems, const Accum &acc
         }
         return LUTGEMM_OK;
     }
-    // Share the launch's workgroup budget in proportion to each problem's sign bytes.
+    // Share the launch's workgroup budget so that the longest range of every problem takes about
+    // the same time.  An item costs a table build plus look-ups in proportion to its bit planes
+    // (0.45 + 0.13 * nb us measured), whatever the problem; the launch ends with its slowest
+    // workgroup, so the items per workgroup of problem i are floor(T / cost_i) for the smallest T
+    // whose workgroups fit the budget.  (Sharing in proportion to the sign bytes gave q,k,v of
+    // 2, 4 and 3 bits 5, 3 and 4 items per workgroup: 3.6, 2.9 and 3.4 us of work.)
+    // With equal bit widths this is a share in proportion to the items, rounded down: a few
+    // workgroups more than can be resident run as a second, mostly empty round, and fewer
+    // workgroups with more items each are the better trade anyway (q,k,v of 4096x4096 as 3 x 64
+    // workgroups of 4 items 5.31 us per GEMV of the four-launch block, as 3 x 86 of 3 items 5.54).
     const long budget = (long)target_blocks(total_bytes);
+    long items[kMaxGroup];
+    double cost[kMaxGroup];
+    double lo = 0.0, hi = 0.0;
+    for (int i = 0; i < count; ++i) {
+        const Problem &p = g.p[i];
+        items[i] = (long)((p.N + kTileCols - 1) / kTileCols) * p.nsets;
+        cost[i] = 0.45 + 0.13 * p.nb;
+        const double all = (double)items[i] * cost[i];
+        if (all > hi) hi = all;
+    }
+    auto workgroups = [&](double t) {
+        long n = 0;
+        for (int i = 0; i < count; ++i) {
+            long ipw = (long)(t / cost[i]);
+            if (ipw < 1) return (long)1 << 40;
+            n += ((items[i] + ipw - 1) / ipw) * g.p[i].M;
+        }
+        return n;
+    };
+    for (int it = 0; it < 50; ++it) {
+        const double mid = 0.5 * (lo + hi);
+        if (workgroups(mid) <= budget) hi = mid; else lo = mid;
+    }
     int begin = 0;
     bool any_split = false;
     for (int i = 0; i < count; ++i) {
         Problem &p = g.p[i];
-        const long mine = (long)p.N * (p.K / 8) * p.nb * p.M;
-        // (rounded down: a few workgroups more than can be resident run as a second, mostly
-        // empty round, and fewer workgroups with more items each are the better trade anyway:
-        // q,k,v of 4096x4096 as 3 x 64 workgroups of 4 items 5.31 us per GEMV of the four-launch
-        // block, as 3 x 86 of 3 items 5.54)
-        long want = budget * mine / (total_bytes > 0 ? total_bytes : 1);
-        if (want < 1) want = 1;
+        long ipw = (long)(hi / cost[i]);
+        if (ipw < 1) ipw = 1;
+        const long want = ((items[i] + ipw - 1) / ipw) * p.M;
         int rc = plan_lookup(p, 1, want);
         if (rc != LUTGEMM_OK) return rc;
         if (p.n_blocks > begin) begin = p.n_blocks;  // grid.x: the largest problem's workgroups
