@@ -26,8 +26,16 @@
  *           (mv_fp16_bias.hpp:342-380): one more fp16 rounding per eight
  *           inputs, output error about 3e-4 relative instead of 2e-4.)
  *           A NaN input gives NaN and an infinite input gives an infinity
- *           or NaN in every output it reaches, whatever the launch plan
- *           (partial sums beyond +-65536 count as infinite).
+ *           or NaN in every output it reaches, whatever the launch plan.
+ *           Finite inputs have a guaranteed range: while every partial sum
+ *           over a run of K stays within +-65536, and (calls with two or
+ *           more rows on the look-up kernel, whose tables are fp16) every
+ *           sum of eight |x| stays below 65504, the result is the rounded
+ *           exact sum under every launch plan.  Beyond that range the
+ *           result depends on the plan: a partial sum beyond +-65536 counts
+ *           as infinite where K is split over workgroups and is carried as
+ *           fp32 where it is not, so the same finite problem may give an
+ *           infinity for one M or grouping and a finite value for another.
  * Shape rules enforced here (the reference checks nothing and reads or writes
  * out of bounds instead): K % 32 == 0, N % 4 == 0, 1 <= nb <= 4,
  * 1 <= M <= 65535, 16-byte aligned bW and x, 8-byte aligned row-wise alpha and out.
@@ -240,6 +248,35 @@ typedef struct lutgemm_plan {
 int lutgemm_describe_plan(int format, int N, int K, int nb, int groups, int M, lutgemm_plan *plan);
 
 /*
+ * Tuning options (no counterpart in the reference, whose launch geometry is fixed at
+ * compile time).  Each starts from the environment variable of the same name
+ * (LUTGEMM_TARGET_BLOCKS ...), read once per process; lutgemm_set_option changes it
+ * for every later call of the process (a negative value restores the start value),
+ * lutgemm_get_option reads it.  Results stay within the documented tolerances under
+ * every setting; the options exist for measurements and tests.
+ *   TARGET_BLOCKS : workgroups a look-up launch aims for (0 = 256 up to 24 MB of
+ *                   sign words, 512 beyond: one or two resident workgroups per CU)
+ *   FIRST_SHARE   : per cent of a CU's items its first-dispatched workgroup takes in
+ *                   a 512-workgroup look-up launch (default 60; 50 = equal ranges)
+ *   MFMA_MIN_M    : rows from which a row-wise problem takes the matrix-core kernel
+ *                   (default 3; a large value switches that kernel off)
+ *   MFMA_BLOCKS   : workgroups aimed at per matrix-core launch (0 = the cost model)
+ *   PAIR_TABLES   : 1 = two rows share one table set of fp16 pairs on the look-up
+ *                   kernel, 0 = one fp32 table set per row
+ *   SINGLE_ITEM   : 1 = launches whose ranges all hold one item take the kernel
+ *                   instance that requests nothing beyond it, 0 = the general one
+ */
+#define LUTGEMM_OPTION_TARGET_BLOCKS 0
+#define LUTGEMM_OPTION_FIRST_SHARE 1
+#define LUTGEMM_OPTION_MFMA_MIN_M 2
+#define LUTGEMM_OPTION_MFMA_BLOCKS 3
+#define LUTGEMM_OPTION_PAIR_TABLES 4
+#define LUTGEMM_OPTION_SINGLE_ITEM 5
+#define LUTGEMM_OPTION_COUNT 6
+int lutgemm_set_option(int which, int value);
+int lutgemm_get_option(int which);
+
+/*
  * Measurement helpers for the floors any kernel of this library sits on (no
  * counterpart in the reference): a kernel that streams `bytes` (multiple of 16)
  * from `src` with the same 128-bit non-temporal loads as the look-up kernel and
@@ -288,13 +325,20 @@ int lutgemm_release_workspaces(void);
  *                            receives, spread over a row's slots, the sum of the
  *                            squares of the row's final outputs;
  *   the consuming problem takes x_f16 = that next_input, K = that N, and
- *     sumsq_in_f32 / sumsq_in_slots : that array (16-byte aligned) and its N/32 slots per row:
+ *     sumsq_in_f32 / sumsq_in_slots : that array (16-byte aligned) and its slots per row,
+ *                            which must be K / 32 (LUTGEMM_EINVAL otherwise):
  *                            y = rsqrt(sum(slots) / K + norm_eps) * W x.
  *   All five may be NULL / 0; next_norm_weight and next_input come together;
  *   sumsq_in excludes norm_weight_f16.  Which slot receives which columns is
- *   unspecified; a slot normally receives one float add (two when outputs of a
- *   32-column run were completed by different workgroups), so the sums are
- *   reproducible from run to run.
+ *   unspecified.  On the look-up kernel a slot normally receives one float add
+ *   (two when outputs of a 32-column run were completed by different
+ *   workgroups), and two adds commute, so the sums are reproducible from run to
+ *   run; on the matrix-core kernel with K cut into three or more slices a slot
+ *   may receive that many adds in arrival order, and the sums (hence the
+ *   consuming problem's outputs) may differ in the last bits between runs.
+ *   Nothing a problem of the call writes (out, next_input, sumsq_out) may overlap
+ *   what another write or a read (x, gate, sumsq_in) of the same call touches
+ *   (LUTGEMM_EINVAL).
  */
 typedef struct lutgemm_fused_problem {
     const uint32_t *bW;

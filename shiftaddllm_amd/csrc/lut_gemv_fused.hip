@@ -24,7 +24,7 @@ template <int NB>
 hipError_t launch_nb(const Problem &p, int xform, hipStream_t stream)
 {
     const dim3 grid((unsigned)p.wgs_per_chunk, (unsigned)p.mchunks), block(kThreads);
-    static const bool single_item = !(getenv("LUTGEMM_SINGLE_ITEM") && *getenv("LUTGEMM_SINGLE_ITEM") == '0');
+    const bool single_item = option(LUTGEMM_OPTION_SINGLE_ITEM) != 0;
     if (p.items_per_wg == 1 && p.short_items == 1 && single_item) {
         if (xform == kXNorm)
             hipLaunchKernelGGL((lut_gemv_fused_kernel<NB, kXNorm, true>), grid, block, 0, stream, p);

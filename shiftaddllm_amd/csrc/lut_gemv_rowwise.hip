@@ -8,19 +8,15 @@
 namespace lutgemm {
 namespace {
 
-// Rows are taken two at a time through tables whose entries hold both rows as fp16
-// halves; LUTGEMM_PAIR_TABLES=0 keeps one fp32 table set per row.
-bool pair_tables_enabled()
-{
-    const char *v = getenv("LUTGEMM_PAIR_TABLES");
-    return !(v && *v == '0');
-}
-
 template <int NB, int MODE>
 hipError_t launch_nb(const Problem &p, int mrows, hipStream_t stream)
 {
-    static const bool pair_tables = pair_tables_enabled();
-    static const bool single_item = !(getenv("LUTGEMM_SINGLE_ITEM") && *getenv("LUTGEMM_SINGLE_ITEM") == '0');
+    // Rows are taken two at a time through tables whose entries hold both rows as fp16 halves
+    // unless LUTGEMM_OPTION_PAIR_TABLES is 0 (one fp32 table set per row then); launches whose
+    // ranges all hold one item take the instance that requests nothing for a second item unless
+    // LUTGEMM_OPTION_SINGLE_ITEM is 0.
+    const bool pair_tables = option(LUTGEMM_OPTION_PAIR_TABLES) != 0;
+    const bool single_item = option(LUTGEMM_OPTION_SINGLE_ITEM) != 0;
     const dim3 grid((unsigned)p.wgs_per_chunk, (unsigned)p.mchunks), block(kThreads);
     if (mrows == 4 && pair_tables)
         hipLaunchKernelGGL((lut_gemv_kernel<NB, MODE, 4, true>), grid, block, 0, stream, p);

@@ -5,6 +5,7 @@
 #include <stdint.h>
 #include <stdlib.h>
 
+#include <atomic>
 #include <map>
 #include <mutex>
 #include <utility>
@@ -129,7 +130,26 @@ int env_int(const char *name, int fallback)
     return (v && *v) ? atoi(v) : fallback;
 }
 
-// Tuning knob (read once): LUTGEMM_TARGET_BLOCKS = workgroups a look-up launch aims
+// Tuning options (lutgemm_set_option): each starts from its environment variable, read once.
+struct Option {
+    const char *env;
+    int fallback;
+};
+constexpr Option kOptions[LUTGEMM_OPTION_COUNT] = {
+    {"LUTGEMM_TARGET_BLOCKS", 0}, {"LUTGEMM_FIRST_SHARE", 60}, {"LUTGEMM_MFMA_MIN_M", 3},
+    {"LUTGEMM_MFMA_BLOCKS", 0},   {"LUTGEMM_PAIR_TABLES", 1},  {"LUTGEMM_SINGLE_ITEM", 1},
+};
+std::atomic<int> g_option[LUTGEMM_OPTION_COUNT];
+std::once_flag g_option_once;
+
+void load_options()
+{
+    std::call_once(g_option_once, [] {
+        for (int i = 0; i < LUTGEMM_OPTION_COUNT; ++i) g_option[i].store(env_int(kOptions[i].env, kOptions[i].fallback));
+    });
+}
+
+// LUTGEMM_OPTION_TARGET_BLOCKS = workgroups a look-up launch aims
 // for.  74 KiB of LDS per workgroup lets two be resident per CU, and a launch above
 // what is resident at once runs a second, mostly empty round that costs as much as
 // the first.
@@ -144,7 +164,7 @@ int env_int(const char *name, int fallback)
 // 1.6 items per workgroup, 5.91 vs 6.37).
 int target_blocks(long sign_bytes, long items = 0, bool block_alpha = false)
 {
-    static const int v = env_int("LUTGEMM_TARGET_BLOCKS", 0);
+    const int v = option(LUTGEMM_OPTION_TARGET_BLOCKS);
     if (v > 0) return v;
     if (block_alpha && items > 4 * 256) return 512;
     return sign_bytes <= (24l << 20) ? 256 : 512;  // 1 or 2 workgroups x 256 CUs
@@ -159,8 +179,7 @@ int target_blocks(long sign_bytes, long items = 0, bool block_alpha = false)
 // items fill the CUs better than 360 of 3), 8192x8192x4 unchanged.
 int first_share()
 {
-    static const int v = env_int("LUTGEMM_FIRST_SHARE", 60);
-    return v;
+    return option(LUTGEMM_OPTION_FIRST_SHARE);
 }
 
 // Cut the (tile, set) items of a problem into contiguous ranges, one per workgroup,
@@ -266,8 +285,7 @@ int fill_problem(Problem &p, int mode, const uint32_t *bW, const void *alpha, co
 
 int mfma_min_rows()
 {
-    static const int v = env_int("LUTGEMM_MFMA_MIN_M", 3);
-    return v;
+    return option(LUTGEMM_OPTION_MFMA_MIN_M);
 }
 
 // The matrix-core path needs whole 128-input steps inside one alpha group and
@@ -304,8 +322,7 @@ void plan_mfma(Problem &p, int mt, long want)
 // no second one).  Measured, 8192x8192x4: 36.4 us at 256 and 40.0 at 512.
 int mfma_blocks_override()
 {
-    static const int v = env_int("LUTGEMM_MFMA_BLOCKS", 0);
-    return v;
+    return option(LUTGEMM_OPTION_MFMA_BLOCKS);
 }
 
 // K-slices per tile for the problems of one launch (all get the same number, each up to
@@ -481,6 +498,9 @@ int run_group(int count, const lutgemm_fused_problem *problems, const Accum &acc
         if (q.sumsq_out_f32 && q.N % 32 != 0) return LUTGEMM_EINVAL;
         if (q.sumsq_in_f32 && (q.sumsq_in_slots <= 0 || q.norm_weight_f16 || !(q.norm_eps >= 0.0f))) return LUTGEMM_EINVAL;
         if (!q.sumsq_in_f32 && q.sumsq_in_slots != 0) return LUTGEMM_EINVAL;
+        // the slots are those a completing problem of K outputs fills (one per 32 columns); the
+        // matrix-core kernel reads them four at a time
+        if (q.sumsq_in_f32 && (q.K % 32 != 0 || q.sumsq_in_slots != q.K / 32)) return LUTGEMM_EINVAL;
         if (!aligned(q.next_input_f16, 2) || !aligned(q.next_norm_weight_f16, 2) || !aligned(q.sumsq_out_f32, 4) ||
             !aligned(q.sumsq_in_f32, 16))
             return LUTGEMM_EALIGN;
@@ -498,14 +518,34 @@ int run_group(int count, const lutgemm_fused_problem *problems, const Accum &acc
         words += (size_t)q.M * q.N;
         total_bytes += (long)q.N * (q.K / 8) * q.nb * q.M;
     }
-    // every problem finishes its outputs with a plain read-modify-write: two problems
-    // of one launch may not write the same memory
-    for (int i = 0; i < count; ++i)
-        for (int j = i + 1; j < count; ++j) {
-            const char *a0 = (const char *)g.p[i].out, *a1 = a0 + (size_t)g.p[i].M * g.p[i].N * 2;
-            const char *b0 = (const char *)g.p[j].out, *b1 = b0 + (size_t)g.p[j].M * g.p[j].N * 2;
-            if (a0 < b1 && b0 < a1) return LUTGEMM_EINVAL;
+    // Every problem finishes its outputs with a plain read-modify-write, and the outputs are
+    // requested early: nothing a problem of the launch writes (out, next_input, sumsq_out) may
+    // overlap anything another write or a read of the launch (x, gate) touches.
+    {
+        struct Span {
+            const char *lo, *hi;
+            bool written;
+        };
+        Span spans[6 * kMaxGroup];
+        int n = 0;
+        auto add = [&](const void *ptr, size_t bytes, bool written) {
+            if (ptr) spans[n++] = Span{(const char *)ptr, (const char *)ptr + bytes, written};
+        };
+        for (int i = 0; i < count; ++i) {
+            const Problem &p = g.p[i];
+            const size_t mn = (size_t)p.M * p.N, mk = (size_t)p.M * p.K;
+            add(p.out, mn * 2, true);
+            add(p.next_in, mn * 2, true);
+            add(p.sumsq_out, (size_t)p.M * (p.N / 32) * 4, true);
+            add(p.x, mk * 2, false);
+            add(p.gate, mk * 2, false);
+            add(p.sumsq_in, (size_t)p.M * p.sumsq_slots * 4, false);
         }
+        for (int i = 0; i < n; ++i)
+            for (int j = i + 1; j < n; ++j)
+                if ((spans[i].written || spans[j].written) && spans[i].lo < spans[j].hi && spans[j].lo < spans[i].hi)
+                    return LUTGEMM_EINVAL;
+    }
     // The matrix-core kernel takes plain and (as a group launch) overwriting problems.
     // Input transforms stay with the look-up kernel: there a workgroup transforms only
     // its K-slice of one row, while every 64-output workgroup of the matrix-core kernel
@@ -621,6 +661,12 @@ using namespace lutgemm;
 
 int lutgemm_internal_hip_fail(int hip_error) { return hip_fail((hipError_t)hip_error); }
 
+int lutgemm::option(int which)
+{
+    load_options();
+    return g_option[which].load(std::memory_order_relaxed);
+}
+
 extern "C" {
 
 const char *lutgemm_strerror(int code)
@@ -644,6 +690,20 @@ const char *lutgemm_strerror(int code)
 }
 
 int lutgemm_last_hip_error(void) { return g_last_hip_error; }
+
+int lutgemm_set_option(int which, int value)
+{
+    if (which < 0 || which >= LUTGEMM_OPTION_COUNT) return LUTGEMM_EINVAL;
+    load_options();
+    g_option[which].store(value < 0 ? env_int(kOptions[which].env, kOptions[which].fallback) : value);
+    return LUTGEMM_OK;
+}
+
+int lutgemm_get_option(int which)
+{
+    if (which < 0 || which >= LUTGEMM_OPTION_COUNT) return LUTGEMM_EINVAL;
+    return option(which);
+}
 
 int lutgemm_gemv_rowwise_f16(const uint32_t *bW, const void *alpha_f16, const void *x_f16,
                              void *out_f16, int N, int K, int nb, int num_groups, int M,

@@ -7,6 +7,9 @@
 
 namespace lutgemm {
 
+// current value of a tuning option (LUTGEMM_OPTION_* of the public header)
+int option(int which);
+
 // look-up kernel, one problem; grid = (p.wgs_per_chunk, p.mchunks); mrows in {1, 2, 4}
 hipError_t launch_gemv_rowwise(const Problem &p, int mode, int mrows, hipStream_t stream);       // kRowF16, kUniformF16
 hipError_t launch_gemv_block(const Problem &p, int mode, int mrows, hipStream_t stream);         // kBlock*

@@ -33,6 +33,8 @@ C_ABI_SYMBOLS = (
     "lutgemm_workspace_words",
     "lutgemm_reserve_workspace",
     "lutgemm_describe_plan",
+    "lutgemm_set_option",
+    "lutgemm_get_option",
     "lutgemm_measure_stream_read",
     "lutgemm_measure_empty_launch",
     "lutgemm_release_workspaces",
@@ -43,6 +45,7 @@ C_ABI_SYMBOLS = (
 
 
 MAX_GROUP = 8
+OPTIONS = {"TARGET_BLOCKS": 0, "FIRST_SHARE": 1, "MFMA_MIN_M": 2, "MFMA_BLOCKS": 3, "PAIR_TABLES": 4, "SINGLE_ITEM": 5}
 NOALLOC_MAX_WORDS = 1 << 18
 
 
@@ -132,6 +135,10 @@ def cabi() -> ctypes.CDLL:
         lib.lutgemm_copy_bytes.restype = ci
         lib.lutgemm_describe_plan.argtypes = [ci, ci, ci, ci, ci, ci, ctypes.POINTER(Plan)]
         lib.lutgemm_describe_plan.restype = ci
+        lib.lutgemm_set_option.argtypes = [ci, ci]
+        lib.lutgemm_set_option.restype = ci
+        lib.lutgemm_get_option.argtypes = [ci]
+        lib.lutgemm_get_option.restype = ci
         lib.lutgemm_workspace_words.argtypes = [ci, ci]
         lib.lutgemm_workspace_words.restype = sz
         lib.lutgemm_reserve_workspace.argtypes = [vp, sz]

@@ -88,6 +88,43 @@ def test_malformed_calls_are_rejected_on_the_host(lib):
     assert lib.lutgemm_copy_bytes(p, p, 0, None) == 0
 
 
+def test_fused_call_rejects_bad_split_norm_slots_and_overlapping_operands(lib):
+    # Host-side validation only: every call below must fail before anything is launched.
+    from shiftaddllm_amd import native
+    E_INVAL = -1
+    base = 0x100000
+
+    def problem(M=8, K=256, N=256, **kw):
+        f = dict(bW=base, alpha_f16=base + 0x10000, x_f16=base + 0x20000, out_f16=base + 0x30000, N=N, K=K, nb=2,
+                 num_groups=K // 128, M=M, overwrite=0, norm_weight_f16=None, gate_f16=None, norm_eps=1e-5,
+                 next_norm_weight_f16=None, next_input_f16=None, sumsq_out_f32=None, sumsq_in_f32=None,
+                 sumsq_in_slots=0)
+        f.update(kw)
+        return native.FusedProblem(**f)
+
+    def call(*problems):
+        arr = (native.FusedProblem * len(problems))(*problems)
+        return lib.lutgemm_gemv_rowwise_f16_fused(len(problems), arr, None)
+
+    sums = base + 0x40000
+    # the slots of the consuming side are K / 32, whatever kernel the row count selects
+    for M in (1, 8):
+        assert call(problem(M=M, sumsq_in_f32=sums, sumsq_in_slots=1)) == E_INVAL
+        assert call(problem(M=M, sumsq_in_f32=sums, sumsq_in_slots=6)) == E_INVAL
+        assert call(problem(M=M, sumsq_in_f32=sums, sumsq_in_slots=9)) == E_INVAL
+    assert call(problem(sumsq_in_f32=None, sumsq_in_slots=8)) == E_INVAL
+    # outputs of two problems overlap
+    assert call(problem(), problem(bW=base + 0x50000)) == E_INVAL
+    # next_input of one problem is the input of another problem of the same call
+    nw = base + 0x60000
+    assert call(problem(next_norm_weight_f16=nw, next_input_f16=base + 0x70000),
+                problem(x_f16=base + 0x70000, out_f16=base + 0x80000)) == E_INVAL
+    # two problems share a row of sums of squares
+    assert call(problem(sumsq_out_f32=sums), problem(out_f16=base + 0x80000, sumsq_out_f32=sums)) == E_INVAL
+    # an output is another problem's gate row
+    assert call(problem(gate_f16=base + 0x90000), problem(out_f16=base + 0x80000, gate_f16=base + 0x30000)) == E_INVAL
+
+
 def test_python_module_exposes_reference_signatures():
     from shiftaddllm_amd import native
     if not os.path.exists(native.TORCH_EXT):

@@ -301,3 +301,82 @@ def test_split_rmsnorm_with_swiglu_input_and_bad_arguments(gpu_device):
     lin_odd = _random_lin(gpu_device, 528, K, 2, 9)
     x_odd = torch.zeros((M, 528), dtype=torch.float16, device=gpu_device)
     assert _split_call(lib, lin_odd, up, x_odd, M, sumsq_out=sumsq) == -1
+
+
+# ---- the fused entry point directly against the oracle on numpy-transformed inputs ------
+
+def _np_lin(lin):
+    return lin[0].cpu().numpy(), lin[1].cpu().numpy()
+
+
+@pytest.mark.parametrize("M", [1, 2])
+def test_fused_norm_gate_and_overwrite_against_the_oracle(gpu_device, M):
+    """RMSNorm input, SiLU(gate) * x input and overwrite, each checked against the scalar oracle fed
+    with inputs transformed in numpy (nothing of the library on the reference side)."""
+    import numpy as np
+    import oracle as orc
+    lib = native.cabi()
+    K, N, eps = 2048, 768, 1e-5
+    g = torch.Generator(device=gpu_device).manual_seed(900 + M)
+    x = (torch.randn((M, K), generator=g, device=gpu_device) * 2.5).half()
+    w = (1 + 0.2 * torch.randn((K,), generator=g, device=gpu_device)).half()
+    gate = (torch.randn((M, K), generator=g, device=gpu_device) * 2).half()
+    lin = _random_lin(gpu_device, N, K, 3, 17)
+    bW, alpha = _np_lin(lin)
+    xn, wn, gn = x.cpu().numpy().astype(np.float32), w.cpu().numpy().astype(np.float32), gate.cpu().numpy().astype(np.float32)
+
+    # RMSNorm folded in: tables of fp16(x * weight), sums scaled by the row's reciprocal RMS; overwrite
+    got = torch.full((M, N), float("nan"), dtype=torch.float16, device=gpu_device)
+    _ok(_fused_call(lib, [lin], x, [got], norm=w, overwrite=True, eps=eps))
+    torch.cuda.synchronize()
+    h = (xn * wn).astype(np.float16)
+    _, y32 = orc.gemv_rowwise_c(bW, alpha, h, K // 128)
+    scale = 1.0 / np.sqrt((xn.astype(np.float64) ** 2).mean(-1, keepdims=True) + eps)
+    rel, mad = orc.error_metrics(got.float().cpu().numpy(), (y32 * scale).astype(np.float32))
+    assert rel <= 2e-3 and mad <= 1e-2, ("norm", rel, mad)
+
+    # SiLU(gate) * x with the roundings of the separate fp16 operations; accumulates into a residual
+    res = torch.randn((M, N), generator=g, device=gpu_device).half()
+    got = res.clone()
+    _ok(_fused_call(lib, [lin], x, [got], gate=gate))
+    torch.cuda.synchronize()
+    silu = (gn / (1.0 + np.exp(-gn))).astype(np.float16).astype(np.float32)
+    act = (silu * xn).astype(np.float16)
+    want, _ = orc.gemv_rowwise_c(bW, alpha, act, K // 128, out=res.cpu().numpy())
+    rel, mad = orc.error_metrics(got.float().cpu().numpy(), want.astype(np.float32))
+    assert rel <= 2e-3 and mad <= 1e-2, ("gate", rel, mad)
+
+
+@pytest.mark.parametrize("M", [1, 8])                        # look-up kernel, matrix-core kernel
+def test_split_norm_fields_against_the_oracle(gpu_device, M):
+    """Completing side: out += W a, next_input = fp16(out * weight), sums of squares of out.
+    Consuming side: y = rsqrt(sum / K + eps) * W next_input.  Both against the scalar oracle."""
+    import numpy as np
+    import oracle as orc
+    lib = native.cabi()
+    K, N, N2, eps = 1024, 2048, 512, 1e-5
+    g = torch.Generator(device=gpu_device).manual_seed(950 + M)
+    a = torch.randn((M, K), generator=g, device=gpu_device).half()
+    res = (torch.randn((M, N), generator=g, device=gpu_device) * 3).half()
+    w = (1 + 0.2 * torch.randn((N,), generator=g, device=gpu_device)).half()
+    lin1, lin2 = _random_lin(gpu_device, N, K, 3, 23), _random_lin(gpu_device, N2, N, 2, 29)
+
+    x = res.clone()
+    nxt = torch.full((M, N), 7.0, dtype=torch.float16, device=gpu_device)
+    sumsq = torch.zeros((M, N // 32), dtype=torch.float32, device=gpu_device)
+    _ok(_split_call(lib, lin1, a, x, M, next_norm=w, next_in=nxt, sumsq_out=sumsq))
+    y = torch.full((M, N2), float("nan"), dtype=torch.float16, device=gpu_device)
+    _ok(_split_call(lib, lin2, nxt, y, M, overwrite=True, sumsq_in=sumsq))
+    torch.cuda.synchronize()
+
+    want_x, _ = orc.gemv_rowwise_c(*_np_lin(lin1), a.cpu().numpy(), K // 128, out=res.cpu().numpy())
+    rel, mad = orc.error_metrics(x.float().cpu().numpy(), want_x.astype(np.float32))
+    assert rel <= 2e-3 and mad <= 1e-2, ("completing", rel, mad)
+    # derived from the outputs the GPU rounded: exact
+    xg = x.cpu().numpy().astype(np.float32)
+    assert np.array_equal(nxt.cpu().numpy(), (xg * w.cpu().numpy().astype(np.float32)).astype(np.float16))
+    np.testing.assert_allclose(sumsq.sum(-1).cpu().numpy(), (xg.astype(np.float64) ** 2).sum(-1), rtol=1e-5)
+    _, y32 = orc.gemv_rowwise_c(*_np_lin(lin2), nxt.cpu().numpy(), N // 128)
+    scale = 1.0 / np.sqrt((xg.astype(np.float64) ** 2).sum(-1, keepdims=True) / N + eps)
+    rel, mad = orc.error_metrics(y.float().cpu().numpy(), (y32 * scale).astype(np.float32))
+    assert rel <= 2e-3 and mad <= 1e-2, ("consuming", rel, mad)

@@ -77,6 +77,17 @@ def test_config5_small_batches_full_size(gpu_device, N, K, nb, M):
     _assert_close(run_rowwise(gpu_device, bW, alpha, x), want, (N, K, nb, M))
 
 
+@pytest.mark.parametrize("N,K,nb,M", [(28672, 8192, 2, 32), (8192, 28672, 2, 32), (8192, 28672, 4, 16),
+                                      (8192, 28672, 4, 32)])
+def test_config5_long_k_and_wide_cells_at_16_and_32_rows(gpu_device, N, K, nb, M):
+    """The matrix-core plans of the two largest shapes at 16 and 32 rows (224 K-steps per tile on
+    8192 x 28672): a few seconds of scalar oracle each."""
+    print(f"config5 N={N} K={K} nb={nb} M={M}", flush=True)
+    bW, alpha, x = packed_rowwise(N, K, nb, M, seed=N + nb + M)
+    want, _ = orc.gemv_rowwise_c(bW.numpy(), alpha.numpy(), x.numpy(), K // 128)
+    _assert_close(run_rowwise(gpu_device, bW, alpha, x), want, (N, K, nb, M))
+
+
 @pytest.mark.parametrize("N,K,nb,group", [(9000, 8224, 4, 32), (13824, 5120, 4, 128), (25604, 4128, 3, 32)])
 def test_ragged_shapes_on_unequal_ranges(gpu_device, N, K, nb, group):
     """More than 24 MB of signs: 512 workgroups whose ranges come in two sizes (the

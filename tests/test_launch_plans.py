@@ -138,3 +138,48 @@ def test_bad_arguments(lib):
     assert lib.lutgemm_describe_plan(ROWWISE, 4096, 4100, 3, 32, 1, ctypes.byref(plan)) == -1   # K % 32
     assert lib.lutgemm_describe_plan(ROWWISE, 4096, 4096, 5, 32, 1, ctypes.byref(plan)) == -1   # bit planes
     assert lib.lutgemm_describe_plan(ROWWISE, 4096, 4096, 3, 32, 0, ctypes.byref(plan)) == -1   # rows
+
+
+def test_tuning_options_change_plans_and_keep_their_invariants(lib):
+    """lutgemm_set_option: every option changes the plan it is documented to change, the plans stay
+    legal, and a negative value restores the start value."""
+    from shiftaddllm_amd import native
+    opt = native.OPTIONS
+    start = {k: lib.lutgemm_get_option(v) for k, v in opt.items()}
+    try:
+        # workgroups a look-up launch aims for
+        _, base = describe(lib, ROWWISE, 11008, 4096, 3, 32, 1)
+        assert base.workgroups <= 256
+        assert lib.lutgemm_set_option(opt["TARGET_BLOCKS"], 512) == 0
+        _, p = describe(lib, ROWWISE, 11008, 4096, 3, 32, 1)
+        assert 256 < p.workgroups <= 512
+        check_plan(p, 11008, 4096, 1)
+        lib.lutgemm_set_option(opt["TARGET_BLOCKS"], -1)
+        # share of the first-dispatched workgroup: 50 = equal ranges
+        _, base = describe(lib, ROWWISE, 28672, 8192, 4, 64, 1)
+        assert base.items_per_long_range > base.items_per_short_range
+        lib.lutgemm_set_option(opt["FIRST_SHARE"], 50)
+        _, p = describe(lib, ROWWISE, 28672, 8192, 4, 64, 1)
+        assert p.items_per_long_range == p.items_per_short_range
+        check_plan(p, 28672, 8192, 1)
+        lib.lutgemm_set_option(opt["FIRST_SHARE"], -1)
+        # rows from which the matrix-core kernel takes over
+        lib.lutgemm_set_option(opt["MFMA_MIN_M"], 2)
+        _, p = describe(lib, ROWWISE, 8192, 8192, 4, 64, 2)
+        assert p.kernel == MATRIX_CORE
+        lib.lutgemm_set_option(opt["MFMA_MIN_M"], 1000)
+        _, p = describe(lib, ROWWISE, 8192, 8192, 4, 64, 16)
+        assert p.kernel == LOOKUP and p.rows_per_pass == 4
+        check_plan(p, 8192, 8192, 16)
+        lib.lutgemm_set_option(opt["MFMA_MIN_M"], -1)
+        # workgroups aimed at per matrix-core launch
+        lib.lutgemm_set_option(opt["MFMA_BLOCKS"], 1024)
+        _, p = describe(lib, ROWWISE, 8192, 8192, 4, 64, 16)
+        assert p.kernel == MATRIX_CORE and p.k_slices == 8
+        check_plan(p, 8192, 8192, 16)
+        lib.lutgemm_set_option(opt["MFMA_BLOCKS"], -1)
+        assert lib.lutgemm_set_option(99, 1) == -1 and lib.lutgemm_get_option(-2) == -1
+    finally:
+        for k, v in opt.items():
+            lib.lutgemm_set_option(v, -1)
+    assert {k: lib.lutgemm_get_option(v) for k, v in opt.items()} == start

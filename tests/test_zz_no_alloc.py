@@ -46,15 +46,22 @@ def test_no_alloc_entry_matches_the_allocating_one_twice_in_a_row(gpu_device):
     dev = gpu_device
     lib = native.cabi()
     stream = torch.cuda.Stream()
-    # K split over many workgroups (accumulator words in use), then a smaller problem
-    # that reuses the first words of the array, then several rows (matrix-core kernel)
-    cases = [(4096, 4096, 3, 1, 11), (1024, 2048, 2, 1, 12), (2048, 1024, 4, 8, 13)]
+    # Every case uses accumulator words (checked through the launch plan): K split over many
+    # workgroups of the look-up kernel, then a smaller problem that reuses the first words of the
+    # array, then two rows through the look-up kernel's pair tables, then several rows on the
+    # matrix-core kernel with K cut into slices, then the first shape again: a call that left a
+    # word dirty would show up in the next one.
+    cases = [(4096, 4096, 3, 1, 11), (1024, 2048, 2, 1, 12), (8192, 4096, 4, 2, 14), (4096, 4096, 3, 8, 13),
+             (4096, 4096, 3, 1, 15)]
     # set-up: the first call on a device resolves the array's address (the runtime places
     # the library's device variables in memory at that moment at the latest)
     w = _operands(dev, 256, 256, 1, 1, 1)
     _call(lib.lutgemm_gemv_rowwise_f16_noalloc, [t.to(dev) for t in w[:3]], w[3].clone().to(dev), stream)
     for (N, K, nb, M, seed) in cases:
         print(f"no-alloc case N={N} K={K} nb={nb} M={M} seed={seed}", flush=True)
+        plan = native.Plan()
+        assert lib.lutgemm_describe_plan(0, N, K, nb, K // 128, M, ctypes.byref(plan)) == 0
+        assert plan.needs_workspace == 1, (N, K, nb, M)
         ops = _operands(dev, N, K, nb, M, seed)
         d = [t.to(dev) for t in ops[:3]]
         out_a, out_b = ops[3].clone().to(dev), ops[3].clone().to(dev)
@@ -62,12 +69,12 @@ def test_no_alloc_entry_matches_the_allocating_one_twice_in_a_row(gpu_device):
         want = _call(lib.lutgemm_gemv_rowwise_f16, d, out_a, stream)
         free_before = torch.cuda.mem_get_info()[0]
         got = _call(lib.lutgemm_gemv_rowwise_f16_noalloc, d, out_b, stream)
-        assert torch.cuda.mem_get_info()[0] == free_before      # nothing was allocated by the call
+        assert torch.cuda.mem_get_info()[0] >= free_before      # nothing was allocated by the call
         assert torch.equal(got.view(torch.int16), want.view(torch.int16)), (N, K, nb, M)
-        # and both agree with the oracle to the bar of the parity suite
+        # and both agree with the oracle to the bar of the parity suite (pair tables: fp16 entries)
         ref, _ = orc.gemv_rowwise_c(ops[0].numpy(), ops[1].numpy(), ops[2].numpy(), K // 128, out=ops[3].numpy())
         rel, mad = orc.error_metrics(got.float().cpu().numpy(), ref.astype(np.float32))
-        assert rel <= 2e-4 and mad <= 1e-3, (rel, mad)
+        assert rel <= (5e-4 if M == 2 else 2e-4) and mad <= 2e-3, (rel, mad)
 
 
 def test_no_alloc_entry_refuses_what_does_not_fit(gpu_device):
