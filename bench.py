@@ -90,6 +90,78 @@ class Gemv:
         return (p(self.bW), p(self.alpha), p(self.x), p(self.out), self.N, self.K, self.nb, self.groups, self.M)
 
 
+def hf_opt_call_path(torch, dev):
+    """The call stack the reference times (model/opt.py:367-423): a HuggingFace OPTForCausalLM
+    (OPT-125m geometry, random weights) whose decoder linears are LutLinear modules in the
+    reference's default storage (int8 exponent triples, 8 row groups, 3 bits), one token per
+    forward with the growing key/value cache, next to the same network with dense fp16 linears.
+    Also the host time of one LutLinear.forward (the device is left idle in between)."""
+    try:
+        import transformers
+    except ImportError:
+        return {"skipped": "transformers is not importable"}
+    import torch.nn as nn
+    from shiftaddllm_amd import decode
+    from shiftaddllm_amd.lut_gemm.kernel import find_layers
+    from shiftaddllm_amd.lut_gemm.quant import LutLinear, make_lut
+
+    cfg = transformers.OPTConfig(vocab_size=50272, hidden_size=768, ffn_dim=3072, num_hidden_layers=12,
+                                 num_attention_heads=12, max_position_embeddings=2048, word_embed_proj_dim=768,
+                                 do_layer_norm_before=True, dropout=0.0)
+    torch.manual_seed(0)
+    dense = transformers.OPTForCausalLM(cfg).half().eval().to(dev)
+    ids = torch.randint(0, cfg.vocab_size, (1, 128), generator=torch.Generator().manual_seed(0))
+    res = {"model": "OPTForCausalLM, OPT-125m geometry (12 x 768, ffn 3072), random init, fp16; 100 warm-up forwards, "
+                    "then 128 single-token forwards with the growing KV cache, sync + wall clock per token, median"}
+    r = decode.benchmark_hf(dense, ids, check=True)
+    res["dense_fp16"] = {"median_ms_per_token": round(r["median_s_per_token"] * 1e3, 4),
+                         "tokens_per_s": round(r["tokens_per_s"], 1), "ppl": round(r["ppl"], 1)}
+    nb, R = 3, 8
+    g = torch.Generator(device=dev).manual_seed(1)
+    count = 0
+    for layer in dense.model.decoder.layers:
+        names = find_layers(layer, layers=(nn.Linear,))
+        for name, lin in names.items():
+            K = lin.in_features
+            make_lut(layer, {name: None}, wbit=nb, group_size=K // R)     # num_groups = K // group_size = R row groups
+        for mod in find_layers(layer, layers=(LutLinear,)).values():
+            mod.to(dev)
+            mod.binaryWeight.data = torch.randint(-2 ** 31, 2 ** 31 - 1, mod.binaryWeight.shape, generator=g, device=dev,
+                                                  dtype=torch.int32)
+            code = torch.full(mod.alpha.shape, -128, dtype=torch.int8, device=dev)
+            e = torch.randint(-9, -6, mod.alpha.shape[:-1], generator=g, device=dev) \
+                - torch.arange(nb, device=dev).view(1, nb, 1)
+            code[..., 0] = e.to(torch.int8)
+            mod.alpha.data = code
+            count += 1
+    lut = dense
+    for reuse in (False, True):
+        for mod in find_layers(lut, layers=(LutLinear,)).values():
+            mod.reuse_output = reuse
+        r = decode.benchmark_hf(lut, ids, check=True)
+        res["lut_reused_output_buffers" if reuse else "lut"] = {
+            "median_ms_per_token": round(r["median_s_per_token"] * 1e3, 4), "tokens_per_s": round(r["tokens_per_s"], 1),
+            "ppl": round(r["ppl"], 1)}
+    res["lut_linears"] = count
+    # host time of one LutLinear.forward: calls back to back without synchronising would queue,
+    # so time a burst and divide (the kernels, 4-5 us each, are shorter than the host path)
+    mod = lut.model.decoder.layers[0].fc1
+    mod.reuse_output = False
+    x = torch.randn((1, 1, mod.K), device=dev).half()
+    for _ in range(50):
+        mod(x)
+    torch.cuda.synchronize()
+    t = time.perf_counter()
+    for _ in range(500):
+        mod(x)
+    host = (time.perf_counter() - t) / 500
+    torch.cuda.synchronize()
+    res["lutlinear_forward_host_us"] = round(host * 1e6, 2)
+    del lut, dense
+    torch.cuda.empty_cache()
+    return res
+
+
 def main():
     args = parse_args()
     if args.gpus != 1:
@@ -608,6 +680,11 @@ def main():
                                 "residual row and the GEMVs that read it, SiLU*up as a HIP kernel "
                                 "(6 launches per block); embedding gather and fp16 lm_head in torch")
 
+    # ---- the reference's real call path: HF OPT -> LutLinear.forward -> lutgemm_compute_block_shiftInt8 ----
+    hf_res = None
+    if not (args.no_decode or args.plain_only):
+        hf_res = hf_opt_call_path(torch, dev)
+
     traffic = None
     if os.path.exists(TRAFFIC_NOTE):
         for line in open(TRAFFIC_NOTE):
@@ -649,6 +726,7 @@ def main():
         "cpu_baseline": cpu,
         "fused_launches": fused,
         "decode": decode_res,
+        "hf_opt_call_path": hf_res,
         "configs": configs,
         "parity": parity,
         "pool_build_s": round(t_pool, 2),

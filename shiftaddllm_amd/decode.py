@@ -369,11 +369,14 @@ class LutDecoder(nn.Module):
 
 
 @torch.no_grad()
-def benchmark(model: LutDecoder, input_ids: torch.Tensor, generate: int = 128, warmup: int = 10):
+def benchmark(model: LutDecoder, input_ids: torch.Tensor, generate: int = 128, warmup: int = 10, check: bool = False):
     """input_ids [B, T] prompt.  Every prompt token, then `generate` greedy tokens,
     is one synchronised single-token step.  Returns a dict with the median seconds
     per token over the generated tokens (and over the prompt tokens), tokens/s
-    (batch * 1/median) and the generated ids."""
+    (batch * 1/median) and the generated ids.  With `check` the cross-entropy of every
+    prompt position's logits against the next prompt token is accumulated as well and
+    `ppl` = exp(mean loss) is returned, as model/opt.py:382-384,414-423 does (outside
+    the timed region of a token)."""
     B, T = input_ids.shape
     assert B == model.batch and T + generate <= model.cfg.max_positions
     dev = model.ids.device
@@ -384,6 +387,7 @@ def benchmark(model: LutDecoder, input_ids: torch.Tensor, generate: int = 128, w
     model.reset()
     times_prompt, times_gen, out_ids = [], [], []
     nxt = None
+    tot = torch.zeros((), dtype=torch.float32, device=dev)
     for i in range(T + generate):
         ids = input_ids[:, i] if i < T else nxt
         torch.cuda.synchronize()
@@ -391,14 +395,53 @@ def benchmark(model: LutDecoder, input_ids: torch.Tensor, generate: int = 128, w
         logits = model.forward_token(ids, i)
         torch.cuda.synchronize()
         (times_prompt if i < T else times_gen).append(time.perf_counter() - tick)
+        if check and i < T - 1:
+            tot += F.cross_entropy(logits.float(), input_ids[:, i + 1])
         nxt = logits.argmax(dim=-1)
         if i >= T - 1:
             out_ids.append(nxt.clone())
     med = statistics.median(times_gen) if times_gen else float("nan")
-    return {
+    res = {
         "batch": B, "prompt_tokens": T, "generated_tokens": generate,
         "median_s_per_token": med,
         "median_s_per_prompt_token": statistics.median(times_prompt),
         "tokens_per_s": B / med if med == med else float("nan"),
         "generated": torch.stack(out_ids[:-1], dim=1).cpu() if len(out_ids) > 1 else None,
     }
+    if check:
+        res["ppl"] = float(torch.exp(tot / max(T - 1, 1)).item())
+    return res
+
+
+@torch.no_grad()
+def benchmark_hf(model, input_ids: torch.Tensor, check: bool = False, warmup: int = 100):
+    """The reference's kernel benchmark itself (model/opt.py:367-423) for a HuggingFace
+    causal LM whose linears may be LutLinear: `warmup` single-token forwards of the first
+    token, then every token of input_ids [1, T] is one forward with the growing key/value
+    cache, a device synchronisation and a wall-clock reading; returns the median seconds per
+    token, tokens/s and, with `check`, the perplexity of the sequence under the model."""
+    dev = next(model.parameters()).device
+    input_ids = input_ids.to(dev)
+    T = input_ids.numel()
+    attention_mask = torch.ones((1, T), device=dev)
+    torch.cuda.synchronize()
+    for _ in range(warmup):
+        model(input_ids[:, 0].reshape(1, -1), past_key_values=None, attention_mask=attention_mask[:, :1])
+        torch.cuda.synchronize()
+    past, times = None, []
+    tot = torch.zeros((), dtype=torch.float32, device=dev)
+    for i in range(T):
+        tick = time.perf_counter()
+        out = model(input_ids[:, i].reshape(1, -1), past_key_values=past, attention_mask=attention_mask[:, :i + 1],
+                    use_cache=True)
+        torch.cuda.synchronize()
+        times.append(time.perf_counter() - tick)
+        if check and i != T - 1:
+            tot += F.cross_entropy(out.logits[0].float(), input_ids[:, i + 1])
+        past = out.past_key_values
+        del out
+    med = statistics.median(times)
+    res = {"tokens": T, "median_s_per_token": med, "tokens_per_s": 1.0 / med}
+    if check:
+        res["ppl"] = float(torch.exp(tot / max(T - 1, 1)).item())
+    return res

@@ -107,6 +107,9 @@ class LutLinear(nn.Module):
         self.register_buffer("alpha", a)
         # kept as a plain attribute like the reference (quant.py:28)
         self.bias = bias
+        self.reuse_output = False      # see _output
+        self._bias_cache = None
+        self._out_cache = {}
 
     def quantize_to_apot(self, x):
         return encode_apot_int8(x, self.num_apot)
@@ -122,22 +125,46 @@ class LutLinear(nn.Module):
             state_dict[key] = a[::8].contiguous()
         super()._load_from_state_dict(state_dict, prefix, *args, **kwargs)
 
+    def _bias_rows(self, rows, device):
+        """The bias as `rows` contiguous fp16 rows on `device`, formed once per (rows, device)
+        and per state of the bias tensor: what every call copies its output from."""
+        b = self.bias
+        key = (rows, device, b.data_ptr(), b._version)
+        if self._bias_cache is None or self._bias_cache[0] != key:
+            t = b.detach().to(device=device, dtype=torch.float16).reshape(1, self.N).expand(rows, self.N).contiguous()
+            self._bias_cache = (key, t)
+        return self._bias_cache[1]
+
+    def _output(self, rows, device):
+        """The tensor the kernel accumulates into, pre-filled with the bias (or zeros): a new
+        one per call like the reference's `bias.clone()` (lut_gemm/quant.py:46), or, with
+        `reuse_output`, one buffer per (rows, device) that every call overwrites (no allocation
+        on the call path, e.g. under HIP graph capture; the caller must be done with the previous
+        result)."""
+        if self.reuse_output:
+            buf = self._out_cache.get((rows, device))
+            if buf is None:
+                buf = self._out_cache[(rows, device)] = torch.empty((rows, self.N), dtype=torch.float16, device=device)
+            if self.bias is None:
+                buf.zero_()
+            else:
+                buf.copy_(self._bias_rows(rows, device))
+            return buf
+        if self.bias is None:
+            return torch.zeros((rows, self.N), dtype=torch.float16, device=device)
+        return self._bias_rows(rows, device).clone()
+
     def forward(self, x):
         if x.shape[-1] != self.K:
             raise ValueError(f"expected last dimension {self.K}, got {tuple(x.shape)}")
-        out_shape = list(x.shape)
-        out_shape[-1] = self.N
         dtype = x.dtype
+        # an fp16, contiguous input (what a half-precision decoder passes) goes to the kernel as it is
         x2 = x.reshape(-1, self.K)
-        if x2.dtype != torch.float16:
+        if dtype != torch.float16:
             x2 = x2.to(torch.float16)
-        x2 = x2.contiguous()
-        rows = x2.shape[0]
-        if self.bias is None:
-            output = torch.zeros((rows, self.N), dtype=torch.float16, device=x2.device)
-        else:
-            output = self.bias.detach().to(device=x2.device, dtype=torch.float16).reshape(1, self.N)
-            output = output.expand(rows, self.N).contiguous()
+        if not x2.is_contiguous():
+            x2 = x2.contiguous()
+        output = self._output(x2.shape[0], x2.device)
 
         ext = native.lutgemm
         fmt = self.alpha_format
@@ -153,7 +180,9 @@ class LutLinear(nn.Module):
         else:
             ext.lutgemm_compute_shift_scale(output, self.binaryWeight, self.alpha, x2, self.N,
                                             self.K, self.wbit, self.num_groups)
-        return output.to(dtype).reshape(out_shape)
+        if dtype != torch.float16:
+            output = output.to(dtype)
+        return output.view(*x.shape[:-1], self.N)
 
     def extra_repr(self):
         return "in_features={}, out_features={}, bias={}, wbit={}, group_size={}, alpha_format={}".format(
