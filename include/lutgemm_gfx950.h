@@ -72,6 +72,8 @@ extern "C" {
                                  would have to grow: reserve it beforehand   */
 #define LUTGEMM_ETOOBIG (-7)  /* beyond the fixed buffer of the entry point
                                  that does not allocate                      */
+#define LUTGEMM_ETIMEDOUT (-8) /* lutgemm_chain_status: a wait of a chained
+                                  launch gave up                             */
 
 /* Human-readable text for a return code (static storage). */
 const char *lutgemm_strerror(int code);
@@ -265,6 +267,7 @@ int lutgemm_describe_plan(int format, int N, int K, int nb, int groups, int M, l
  *                   kernel, 0 = one fp32 table set per row
  *   SINGLE_ITEM   : 1 = launches whose ranges all hold one item take the kernel
  *                   instance that requests nothing beyond it, 0 = the general one
+ *   CHAIN_BLOCKS  : workgroups per stage of a chained launch (0 = as TARGET_BLOCKS)
  */
 #define LUTGEMM_OPTION_TARGET_BLOCKS 0
 #define LUTGEMM_OPTION_FIRST_SHARE 1
@@ -272,7 +275,8 @@ int lutgemm_describe_plan(int format, int N, int K, int nb, int groups, int M, l
 #define LUTGEMM_OPTION_MFMA_BLOCKS 3
 #define LUTGEMM_OPTION_PAIR_TABLES 4
 #define LUTGEMM_OPTION_SINGLE_ITEM 5
-#define LUTGEMM_OPTION_COUNT 6
+#define LUTGEMM_OPTION_CHAIN_BLOCKS 6
+#define LUTGEMM_OPTION_COUNT 7
 int lutgemm_set_option(int which, int value);
 int lutgemm_get_option(int which);
 
@@ -358,6 +362,85 @@ typedef struct lutgemm_fused_problem {
 } lutgemm_fused_problem;
 
 int lutgemm_gemv_rowwise_f16_fused(int count, const lutgemm_fused_problem *problems, void *stream);
+
+/*
+ * Row-wise GEMVs that DEPEND on each other in ONE launch (no counterpart in the
+ * reference, which launches every linear layer separately and waits for each).
+ * Of a GEMV's bytes all but the activation row are independent of the GEMV in
+ * front of it, but a launch boundary makes all of them wait: about 2 us of launch
+ * gap, the first memory round trip and the ramp of the stream, per dependent GEMV.
+ * Here up to LUTGEMM_MAX_GROUP problems form one grid; a problem that consumes
+ * another's output requests its sign words and alphas at once and then waits for
+ * the activations only.
+ *
+ * The hand-over goes through TAGGED rows: uint32 [M][N], one word per value =
+ * fp16 bits | tag << 16.  The producer writes every finished value with its tag
+ * (one store past its L2); the consumer re-reads the words it needs until all
+ * carry the tag it expects.  Per problem:
+ *   x_tag    0: x_f16 is plain fp16 [M][K], written before the call;
+ *            t >= 1: x_f16 points at a tagged row uint32 [M][K] and the problem
+ *            waits until the words it needs carry tag t;
+ *   gate_tag the same for gate_f16;
+ *   out_tag  0: out_f16 is plain fp16 [M][N]; t >= 1: a tagged row uint32 [M][N],
+ *            every output is written with tag t (accumulation reads the old
+ *            values whatever their tags).
+ * The other fields of `p` mean what they mean in the fused call (norm_weight:
+ * RMSNorm formed from the row itself, K <= 8192 when it is tagged; gate:
+ * SiLU(gate) * x; overwrite); the split-RMSNorm fields must be NULL / 0
+ * (LUTGEMM_EUNSUP).  1 <= M <= LUTGEMM_CHAIN_MAX_ROWS (one row per workgroup,
+ * look-up kernel).  Tags lie in 1..LUTGEMM_CHAIN_MAX_TAG.
+ *
+ * Order.  Workgroups are dispatched problem by problem in the order given, which
+ * is what keeps a wait from starving the problem it waits for: a problem must
+ * come AFTER every problem of the call whose tag it waits for (LUTGEMM_EINVAL),
+ * and problems must be listed stage by stage (those that wait for nothing, then
+ * those that wait for them, ...).  A tag that no problem of the call writes is
+ * waited for all the same: the row may be written by other work of the process,
+ * but nothing guarantees that such work runs while the call waits, so every wait
+ * is bounded (control->spin_limit_us, 0 = 100000).  A wait that gives up sets bit
+ * 0 of *control->status (device memory, zero before the call); the waiting
+ * workgroups of the call then exit without writing, the kernel ends normally,
+ * and lutgemm_chain_status() reports LUTGEMM_ETIMEDOUT.
+ *
+ * Epoch.  A captured launch is replayed with the same tags, and last replay's
+ * rows would satisfy this replay's waits: the effective tag of base t is
+ * 1 + (t + *control->epoch) % 65535 (epoch: device memory, may be NULL = 0).
+ * Advance the epoch word between replays (lutgemm_chain_advance_epoch, by at
+ * least the number of tag bases in use) so that no row still carries a tag that a
+ * later call waits for before its producer has written it.
+ *
+ * Overlap.  The same tagged row may be written by several problems of a call with
+ * different tags (a residual row that two GEMVs complete one after the other) and
+ * read in between, if the waits order them: a later writer must wait, directly
+ * or through other problems, for the earlier writer and for every reader of the
+ * earlier contents (LUTGEMM_EINVAL otherwise).  Plain rows may not be shared
+ * between a writer and any other problem of the call.
+ * Workspace, capture and error conventions are those of the other entry points.
+ */
+#define LUTGEMM_CHAIN_MAX_ROWS 4
+#define LUTGEMM_CHAIN_MAX_TAG 65534
+typedef struct lutgemm_chain_problem {
+    lutgemm_fused_problem p;
+    int x_tag, gate_tag, out_tag;
+} lutgemm_chain_problem;
+
+typedef struct lutgemm_chain_control {
+    const uint32_t *epoch;
+    uint32_t *status;
+    unsigned spin_limit_us;
+} lutgemm_chain_control;
+
+int lutgemm_gemv_rowwise_f16_chain(int count, const lutgemm_chain_problem *problems,
+                                   const lutgemm_chain_control *control, void *stream);
+
+/* dst_tagged[i] = src_f16[i] | effective tag << 16 (count values), and back. */
+int lutgemm_chain_tag_rows(void *dst_tagged, const void *src_f16, size_t count, int tag, const uint32_t *epoch,
+                           void *stream);
+int lutgemm_chain_untag_rows(void *dst_f16, const void *src_tagged, size_t count, void *stream);
+/* *epoch += by, on the stream. */
+int lutgemm_chain_advance_epoch(uint32_t *epoch, uint32_t by, void *stream);
+/* Synchronises `stream`, reads *status: LUTGEMM_OK or LUTGEMM_ETIMEDOUT. */
+int lutgemm_chain_status(const uint32_t *status, void *stream);
 
 /*
  * ---- decode-step glue (no counterpart in the reference) ----------------------

@@ -46,7 +46,7 @@ def _run(cmd):
 
 
 KERNEL_SOURCES = ("lutgemm_host.hip", "lut_gemv_rowwise.hip", "lut_gemv_block.hip", "lut_gemv_block_staged.hip",
-                  "lut_gemv_group.hip", "lut_gemv_fused.hip", "lut_gemm_mfma.hip", "decode_kernels.hip")
+                  "lut_gemv_group.hip", "lut_gemv_fused.hip", "lut_gemv_chain.hip", "lut_gemm_mfma.hip", "decode_kernels.hip")
 KERNEL_HEADERS = ("lutgemm_internal.h", "lutgemm_common.h", "lutgemm_launch.h", "lut_gemv_device.h",
                   "lut_gemm_mfma_device.h")
 

@@ -182,9 +182,17 @@ struct WindowChunk {
     bool live;  // chunks beyond K, or of items beyond the range, read as zero
 };
 
-template <int MROWS, int XF>
-__device__ __forceinline__ WindowChunk fetch_window(const Problem &p, int m0, int set0, int first_rel, int n_items,
-                                                    int tid)
+// Which chunk of the window that starts `first_rel` items into the range thread `tid` fetches:
+// the element offset of its first input in x (and gate), the first input itself (clamped into the
+// row) and whether the chunk is live.
+struct WindowIndex {
+    size_t base;
+    int kc;
+    bool live;
+};
+
+template <int MROWS>
+__device__ __forceinline__ WindowIndex window_index(const Problem &p, int m0, int set0, int first_rel, int n_items, int tid)
 {
     constexpr int kSlots = kWindowSlots / MROWS;  // items per window
     const int c = tid % kTables, slot = (tid / kTables) % kSlots, row = tid / (kTables * kSlots);
@@ -192,16 +200,98 @@ __device__ __forceinline__ WindowChunk fetch_window(const Problem &p, int m0, in
     const int v = set0 + rel;
     const int set = v - fast_div(v, p.by_nsets) * p.nsets;
     const int k0 = (set * kTables + c) * 8;
-    const int kc = min(k0, p.K - 8);
-    const size_t base = (size_t)min(m0 + row, p.M - 1) * p.K + kc;
-    WindowChunk w;
-    w.x = *(const u32x4 *)(p.x + base);
-    w.other = (u32x4){0u, 0u, 0u, 0u};
-    if constexpr (XF == kXGate) w.other = *(const u32x4 *)(p.gate + base);
-    if constexpr (XF == kXNorm) w.other = *(const u32x4 *)(p.norm_w + kc);
-    w.kc = kc;
+    WindowIndex w;
+    w.kc = min(k0, p.K - 8);
+    w.base = (size_t)min(m0 + row, p.M - 1) * p.K + w.kc;
     w.live = k0 < p.K && rel < n_items;
     return w;
+}
+
+template <int MROWS, int XF>
+__device__ __forceinline__ WindowChunk fetch_window(const Problem &p, int m0, int set0, int first_rel, int n_items,
+                                                    int tid)
+{
+    const WindowIndex i = window_index<MROWS>(p, m0, set0, first_rel, n_items, tid);
+    WindowChunk w;
+    w.x = *(const u32x4 *)(p.x + i.base);
+    w.other = (u32x4){0u, 0u, 0u, 0u};
+    if constexpr (XF == kXGate) w.other = *(const u32x4 *)(p.gate + i.base);
+    if constexpr (XF == kXNorm) w.other = *(const u32x4 *)(p.norm_w + i.kc);
+    w.kc = i.kc;
+    w.live = i.live;
+    return w;
+}
+
+// ---- tagged rows (chained launches) ------------------------------------------------------------
+// What a workgroup of a chained launch needs to wait: the launch's epoch, where to report a wait
+// that gave up, and how long a wait may last.
+struct ChainWait {
+    uint32_t epoch;
+    uint32_t *status;
+    long long spin_ticks;
+};
+
+// Read NCH chunks of eight tagged words each (32 bytes at src[c]) until every word of every lane
+// of the wave carries its tag want[c] (already shifted into the upper half); returns the eight
+// fp16 values of each chunk packed into 16 bytes.  Returns false when the wait gave up: the
+// launch's status word is set (by this wave after spin_ticks, or by another wave earlier) and
+// the values are meaningless.  The loads bypass the L2 (agent scope), which other workgroups'
+// stores are written through.  One asm statement holds the requests and their wait: the
+// compiler may place nothing that reads the destination registers in between.
+template <int NCH>
+__device__ __forceinline__ bool poll_tagged(const uint32_t *const (&src)[NCH], const uint32_t (&want)[NCH], u32x4 (&out)[NCH],
+                                            const ChainWait &cw)
+{
+    static_assert(NCH >= 1 && NCH <= 3, "one to three chunks per thread");
+    const long long t0 = wall_clock64();
+    for (;;) {
+        u32x4 lo[NCH], hi[NCH];
+        if constexpr (NCH == 1)
+            asm volatile("global_load_dwordx4 %0, %2, off sc1\n\t"
+                         "global_load_dwordx4 %1, %2, off offset:16 sc1\n\t"
+                         "s_waitcnt vmcnt(0)"
+                         : "=&v"(lo[0]), "=&v"(hi[0]) : "v"(src[0]) : "memory");
+        else if constexpr (NCH == 2)
+            asm volatile("global_load_dwordx4 %0, %4, off sc1\n\t"
+                         "global_load_dwordx4 %1, %4, off offset:16 sc1\n\t"
+                         "global_load_dwordx4 %2, %5, off sc1\n\t"
+                         "global_load_dwordx4 %3, %5, off offset:16 sc1\n\t"
+                         "s_waitcnt vmcnt(0)"
+                         : "=&v"(lo[0]), "=&v"(hi[0]), "=&v"(lo[1]), "=&v"(hi[1]) : "v"(src[0]), "v"(src[1]) : "memory");
+        else
+            asm volatile("global_load_dwordx4 %0, %6, off sc1\n\t"
+                         "global_load_dwordx4 %1, %6, off offset:16 sc1\n\t"
+                         "global_load_dwordx4 %2, %7, off sc1\n\t"
+                         "global_load_dwordx4 %3, %7, off offset:16 sc1\n\t"
+                         "global_load_dwordx4 %4, %8, off sc1\n\t"
+                         "global_load_dwordx4 %5, %8, off offset:16 sc1\n\t"
+                         "s_waitcnt vmcnt(0)"
+                         : "=&v"(lo[0]), "=&v"(hi[0]), "=&v"(lo[1]), "=&v"(hi[1]), "=&v"(lo[2]), "=&v"(hi[2])
+                         : "v"(src[0]), "v"(src[1]), "v"(src[2]) : "memory");
+        uint32_t bad = 0;
+#pragma unroll
+        for (int c = 0; c < NCH; ++c) {
+            const uint32_t w = want[c];
+            bad |= (lo[c].x ^ w) | (lo[c].y ^ w) | (lo[c].z ^ w) | (lo[c].w ^ w) | (hi[c].x ^ w) | (hi[c].y ^ w) |
+                   (hi[c].z ^ w) | (hi[c].w ^ w);
+        }
+        if (__builtin_amdgcn_ballot_w64((bad & 0xffff0000u) != 0) == 0) {
+#pragma unroll
+            for (int c = 0; c < NCH; ++c) {
+                out[c].x = __builtin_amdgcn_perm(lo[c].y, lo[c].x, 0x05040100u);
+                out[c].y = __builtin_amdgcn_perm(lo[c].w, lo[c].z, 0x05040100u);
+                out[c].z = __builtin_amdgcn_perm(hi[c].y, hi[c].x, 0x05040100u);
+                out[c].w = __builtin_amdgcn_perm(hi[c].w, hi[c].z, 0x05040100u);
+            }
+            return true;
+        }
+        if (__hip_atomic_load(cw.status, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u) return false;
+        if (wall_clock64() - t0 > cw.spin_ticks) {
+            if ((threadIdx.x & 63) == 0) __hip_atomic_fetch_or(cw.status, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            return false;
+        }
+        __builtin_amdgcn_s_sleep(2);
+    }
 }
 
 // Transform the chunk and park it in the window.  With a gate row the chunk is
@@ -210,14 +300,35 @@ __device__ __forceinline__ WindowChunk fetch_window(const Problem &p, int m0, in
 // linear in their inputs, so the row's reciprocal RMS is applied to the finished sums
 // instead (flush_tile) and the reduction that yields it is not waited for here.
 // (x * weight is held as fp16: it must stay below 65504.)
+// XF == kXDynamic: the transform is `xf`, known at run time (uniform over the workgroup).
 template <int MROWS, int XF>
-__device__ __forceinline__ void store_window(const WindowChunk &w, float *window, int tid)
+__device__ __forceinline__ void store_window(const WindowChunk &w, float *window, int tid, int xf = XF)
 {
     u32x4 xr = w.x;
     // (opaque: the work on the fetched chunk stays here, after the sign-word requests,
     // instead of being hoisted to where it would have to wait for the chunk first)
     asm volatile("" : "+v"(xr.x), "+v"(xr.y), "+v"(xr.z), "+v"(xr.w));
-    if constexpr (XF != kXNone) {
+    if constexpr (XF == kXDynamic) {
+        if (xf != kXNone) {
+            const u32x4 other = w.other;
+            const uint32_t a[4] = {xr.x, xr.y, xr.z, xr.w};
+            const uint32_t b[4] = {other.x, other.y, other.z, other.w};
+            uint32_t o[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                float v[2];
+#pragma unroll
+                for (int hh = 0; hh < 2; ++hh) {
+                    const float xv = half_bits_to_float((a[j] >> (16 * hh)) & 0xffffu);
+                    const float bv = half_bits_to_float((b[j] >> (16 * hh)) & 0xffffu);
+                    const float silu = half_bits_to_float(float_to_half_bits(__fdividef(bv, 1.0f + __expf(-bv))));
+                    v[hh] = xv * (xf == kXGate ? silu : bv);
+                }
+                o[j] = float_to_half_bits(v[0]) | (float_to_half_bits(v[1]) << 16);
+            }
+            xr = (u32x4){o[0], o[1], o[2], o[3]};
+        }
+    } else if constexpr (XF != kXNone) {
         const u32x4 other = w.other;
         const uint32_t a[4] = {xr.x, xr.y, xr.z, xr.w};
         const uint32_t b[4] = {other.x, other.y, other.z, other.w};
@@ -531,12 +642,22 @@ __device__ __forceinline__ float reduce_scatter_kw(const float (&acc)[4], int kw
 //       range of the launch holds more than that one item (the host's choice).
 // PAIR: rows are taken two at a time through pair tables (fp16 entries; MROWS even,
 //       per-column alphas).
+// DEP: a problem of a chained launch (`cw` non-null): x, gate and out may be tagged rows.  The
+//      operands that depend on nothing (sign words and alphas of the first two items) are
+//      requested at once; the activations are waited for, tag by tag, behind them.
 template <int NB, int MODE, int MROWS, int XF = kXNone, bool EXTRA = false, int ALONE = MROWS == 1 && !is_block(MODE),
-          bool PAIR = false>
-__device__ __forceinline__ void gemv_range(const Problem &p, int range, int mchunk, float *lut)
+          bool PAIR = false, bool DEP = false>
+__device__ __forceinline__ void gemv_range(const Problem &p, int range, int mchunk, float *lut, const ChainWait *cw = nullptr)
 {
     static_assert(!PAIR || (MROWS % 2 == 0 && (MODE == kRowF16 || MODE == kUniformF16)), "pair tables: even row count, per-column alphas");
     static_assert(!(EXTRA || XF == kXNorm) || !is_staged(MODE), "the per-wave sums live in the alpha staging area");
+    static_assert(!DEP || (MROWS == 1 && MODE == kRowF16 && !EXTRA && !PAIR), "chained launches: one row per workgroup, row-wise alphas");
+    static_assert(DEP == (XF == kXDynamic), "chained problems choose their transform at run time, the others at compile time");
+    // the transform: a compile-time constant except for chained problems (one kernel holds them
+    // all, and an instance per bit width and transform is more than the compiler digests: from
+    // eight instances of this function on, it emits an empty kernel)
+    [[maybe_unused]] const int xf = XF != kXDynamic ? XF : p.norm_w ? kXNorm : p.gate ? kXGate : kXNone;
+    constexpr bool kMayNorm = XF == kXNorm || XF == kXDynamic;
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = tid >> 6;
@@ -593,8 +714,10 @@ __device__ __forceinline__ void gemv_range(const Problem &p, int range, int mchu
     constexpr int kSlots = kWindowSlots / MROWS;  // items per window
     const int set0 = set, n_items = rem;
     float *window = stage + kStageDwords;
-    const WindowChunk w0 = fetch_window<MROWS, XF>(p, m0, set0, 0, n_items, tid);
-    constexpr bool kDirectFirst = XF == kXNone && !PAIR;
+    // (a chained problem requests its activations later, behind the first two items' operands)
+    WindowChunk w0;
+    if constexpr (!DEP) w0 = fetch_window<MROWS, XF>(p, m0, set0, 0, n_items, tid);
+    constexpr bool kDirectFirst = XF == kXNone && !PAIR && !DEP;
     // Without an input transform the tables of the first item (row 0) are built straight
     // from a second request for this thread's own chunk, so that nothing but that chunk
     // stands between the start of the kernel and the first table.
@@ -607,14 +730,80 @@ __device__ __forceinline__ void gemv_range(const Problem &p, int range, int mchu
     // fused RMSNorm: every workgroup forms the reciprocal RMS of its rows itself (K
     // fp16 values per row, from L2), requested right behind the window.
     constexpr int kNormChunks = 2;  // 16-byte chunks per thread held in registers: K <= 8192
-    u32x4 nx[XF == kXNorm ? MROWS : 1][kNormChunks];
-    if constexpr (XF == kXNorm) {
+    u32x4 nx[kMayNorm ? MROWS : 1][kNormChunks];
+    if constexpr (XF == kXNorm && !DEP) {
 #pragma unroll
         for (int r = 0; r < MROWS; ++r)
 #pragma unroll
             for (int u = 0; u < kNormChunks; ++u)
                 nx[r][u] = *(const u32x4 *)(xrow[r] + 8 * min(tid + kThreads * u, p.K / 8 - 1));
     }
+    // Chained problem: the activations this thread needs (its chunk of the first window, with a
+    // gate row the same chunk of that, with a norm its share of the whole row), each from a plain
+    // fp16 row (written before the launch) or from a tagged row that an earlier problem of the
+    // launch is still writing.  False when a wait gave up.
+    [[maybe_unused]] uint32_t out_tagw = 0;
+    auto chain_inputs = [&]() -> bool {
+        if constexpr (!DEP) {
+            return true;
+        } else {
+            const WindowIndex wi = window_index<MROWS>(p, m0, set0, 0, n_items, tid);
+            w0.kc = wi.kc;
+            w0.live = wi.live;
+            w0.other = (u32x4){0u, 0u, 0u, 0u};
+            const uint32_t xw = effective_tag(p.x_tag, cw->epoch) << 16;
+            const uint32_t *xt = (const uint32_t *)p.x;  // tagged: one word per value
+            bool ok = true;
+            if (xf == kXNorm) {
+                w0.other = *(const u32x4 *)(p.norm_w + wi.kc);
+                const size_t row0 = (size_t)min(m0, p.M - 1) * p.K;
+                const int c0 = 8 * min(tid, p.K / 8 - 1), c1 = 8 * min(tid + kThreads, p.K / 8 - 1);
+                if (p.x_tag) {
+                    const uint32_t *src[3] = {xt + wi.base, xt + row0 + c0, xt + row0 + c1};
+                    const uint32_t want[3] = {xw, xw, xw};
+                    u32x4 got[3];
+                    ok = poll_tagged<3>(src, want, got, *cw);
+                    w0.x = got[0];
+                    nx[0][0] = got[1];
+                    nx[0][1] = got[2];
+                } else {
+                    w0.x = *(const u32x4 *)(p.x + wi.base);
+                    nx[0][0] = *(const u32x4 *)(p.x + row0 + c0);
+                    nx[0][1] = *(const u32x4 *)(p.x + row0 + c1);
+                }
+            } else if (xf == kXGate) {
+                const uint32_t gw = effective_tag(p.gate_tag, cw->epoch) << 16;
+                const uint32_t *gt = (const uint32_t *)p.gate;
+                if (!p.x_tag) w0.x = *(const u32x4 *)(p.x + wi.base);
+                if (!p.gate_tag) w0.other = *(const u32x4 *)(p.gate + wi.base);
+                if (p.x_tag && p.gate_tag) {
+                    const uint32_t *src[2] = {xt + wi.base, gt + wi.base};
+                    const uint32_t want[2] = {xw, gw};
+                    u32x4 got[2];
+                    ok = poll_tagged<2>(src, want, got, *cw);
+                    w0.x = got[0];
+                    w0.other = got[1];
+                } else if (p.x_tag || p.gate_tag) {
+                    const uint32_t *src[1] = {p.x_tag ? xt + wi.base : gt + wi.base};
+                    const uint32_t want[1] = {p.x_tag ? xw : gw};
+                    u32x4 got[1];
+                    ok = poll_tagged<1>(src, want, got, *cw);
+                    if (p.x_tag) w0.x = got[0]; else w0.other = got[0];
+                }
+            } else {
+                if (p.x_tag) {
+                    const uint32_t *src[1] = {xt + wi.base};
+                    const uint32_t want[1] = {xw};
+                    u32x4 got[1];
+                    ok = poll_tagged<1>(src, want, got, *cw);
+                    w0.x = got[0];
+                } else {
+                    w0.x = *(const u32x4 *)(p.x + wi.base);
+                }
+            }
+            return ok;
+        }
+    };
     // split RMSNorm, consuming side: this thread's share of the rows' sums of squares
     float slot_sum[MROWS];
 #pragma unroll
@@ -634,6 +823,15 @@ __device__ __forceinline__ void gemv_range(const Problem &p, int range, int mchu
     unsigned short out_prev[MROWS];
     auto fetch_out = [&](int t) {
         const int n = min(t * kTileCols + own_col_of(kw), p.N - 1);
+        if constexpr (DEP) {
+            // a tagged row that an earlier problem of the launch may have completed: its values
+            // (whatever their tags) are read past the L2
+            if (p.out_tag) {
+                out_prev[0] = (unsigned short)__hip_atomic_load((const uint32_t *)p.out + (size_t)min(m0, p.M - 1) * p.N + n,
+                                                                __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                return;
+            }
+        }
 #pragma unroll
         for (int r = 0; r < MROWS; ++r)
             out_prev[r] = *((const unsigned short *)(p.out + (size_t)min(m0 + r, p.M - 1) * p.N) + n);
@@ -657,9 +855,10 @@ __device__ __forceinline__ void gemv_range(const Problem &p, int range, int mchu
     // wave's share of the rows' sums of squares in LDS.  The reciprocal RMS is formed
     // from those behind the barrier and is first needed when sums are handed over.
     auto first_window = [&]() {
-        if constexpr (XF == kXNorm) {
+        if constexpr (kMayNorm) {
 #pragma unroll
             for (int r = 0; r < MROWS; ++r) {
+                if (xf != kXNorm) break;
                 float ss = 0.0f;
                 auto add_chunk = [&](const u32x4 &v) {
                     const uint32_t w4[4] = {v.x, v.y, v.z, v.w};
@@ -672,8 +871,9 @@ __device__ __forceinline__ void gemv_range(const Problem &p, int range, int mchu
 #pragma unroll
                 for (int u = 0; u < kNormChunks; ++u)
                     if (tid + kThreads * u < p.K / 8) add_chunk(nx[r][u]);
-                for (int c = tid + kThreads * kNormChunks; c < p.K / 8; c += kThreads)  // K > 8192
-                    add_chunk(*(const u32x4 *)(xrow[r] + 8 * c));
+                if constexpr (!DEP)  // (the host keeps chained norm problems to K <= 8192)
+                    for (int c = tid + kThreads * kNormChunks; c < p.K / 8; c += kThreads)  // K > 8192
+                        add_chunk(*(const u32x4 *)(xrow[r] + 8 * c));
                 ss = wave_sum(ss);
                 if (lane == 0) stage[wave * MROWS + r] = ss;
             }
@@ -693,7 +893,7 @@ __device__ __forceinline__ void gemv_range(const Problem &p, int range, int mchu
                 }
             }
         }
-        store_window<MROWS, XF>(w0, window, tid);
+        store_window<MROWS, XF>(w0, window, tid, xf);
         // (without a transform the first build does not read the window, and the barrier
         // that follows that build publishes the window as well)
         if constexpr (!kDirectFirst) __syncthreads();
@@ -720,7 +920,7 @@ __device__ __forceinline__ void gemv_range(const Problem &p, int range, int mchu
         asm volatile("" : "+v"(kw2));  // (opaque: see own_col_of)
         const int n = t * kTileCols + own_col_of(kw2);
         const bool owner = (kw2 & 1) == 0;
-        bool scaled = XF == kXNorm;
+        bool scaled = xf == kXNorm;
         if constexpr (EXTRA) scaled = scaled || p.sumsq_in != nullptr;
         // the next norm's weight for this lane's column: requested here, used once the
         // sums are complete
@@ -732,6 +932,13 @@ __device__ __forceinline__ void gemv_range(const Problem &p, int range, int mchu
         // with the next norm's weight beside it.
         auto complete = [&](int r, __half *dst, float y) {
             const __half y16 = __float2half_rn(y);
+            if constexpr (DEP) {
+                if (p.out_tag) {
+                    __hip_atomic_store((uint32_t *)p.out + (dst - p.out), out_tagw | (uint32_t)__half_as_ushort(y16),
+                                       __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    return;
+                }
+            }
             *dst = y16;
             if constexpr (EXTRA) {
                 const float yf = __half2float(y16);
@@ -796,8 +1003,9 @@ __device__ __forceinline__ void gemv_range(const Problem &p, int range, int mchu
             // last read): fetch and park the next one.  Not prefetched: ranges of more than
             // a window's items only occur beyond half a billion weights per call, and a
             // conditional load in flight would make every later wait conservative.
+            // (never reached by a chained problem: the host keeps its ranges within one window)
             const WindowChunk w = fetch_window<MROWS, XF>(p, m0, set0, rel, n_items, tid);
-            store_window<MROWS, XF>(w, window, tid);
+            store_window<MROWS, XF>(w, window, tid, xf);
             __syncthreads();
         }
         if constexpr (PAIR) {
@@ -880,7 +1088,40 @@ __device__ __forceinline__ void gemv_range(const Problem &p, int range, int mchu
     int ld_tile = tile, ld_set = set;  // next item to request
     const int pairs = (n_items + 1) / 2;
     auto no_hook = []() {};
-    if constexpr (ALONE == 2) {
+    if constexpr (DEP) {
+        // Chained problem: the first two items' operands are requested at once (the workgroup
+        // may have to wait for its activations anyway, and whatever arrives meanwhile is off
+        // the path that starts when they do); then the activations, tag by tag.
+        load_item<NB, MODE>(opA, p, ld_tile, ld_set, true, kw, q, lane_col, tid);
+        advance(ld_tile, ld_set);
+        load_item<NB, MODE>(opB, p, ld_tile, ld_set, 1 < n_items, kw, q, lane_col, tid);
+        advance(ld_tile, ld_set);
+        __builtin_amdgcn_sched_barrier(0);
+        late_setup();
+        out_tagw = effective_tag(p.out_tag, cw->epoch) << 16;
+        const bool ok = chain_inputs();
+        // every wave leaves its verdict where the others read it behind first_window's barrier:
+        // a workgroup goes on or gives up as a whole
+        if (lane == 0) stage[64 + wave] = ok ? 0.0f : 1.0f;
+        fetch_out(tile);
+        first_window();
+        float gave_up = 0.0f;
+#pragma unroll
+        for (int w = 0; w < kWaves; ++w) gave_up += stage[64 + w];
+        if (gave_up != 0.0f) return;
+        item_step(opA, n_items == 1, no_hook);
+#pragma clang loop unroll(disable)
+        for (int j = 1; j < pairs; ++j) {
+            load_item<NB, MODE>(opA, p, ld_tile, ld_set, true, kw, q, lane_col, tid);
+            advance(ld_tile, ld_set);
+            item_step(opB, false, no_hook);
+            const bool has_b = 2 * j + 1 < n_items;
+            load_item<NB, MODE>(opB, p, ld_tile, ld_set, has_b, kw, q, lane_col, tid);
+            advance(ld_tile, ld_set);
+            item_step(opA, !has_b, no_hook);
+        }
+        if ((n_items & 1) == 0) item_step(opB, true, no_hook);
+    } else if constexpr (ALONE == 2) {
         // One item per range, known at launch: nothing is requested for a second item.  In the
         // general form below a range that ends requests a dummy in place of the item that
         // does not exist (so that every wait can count its loads), and those six to eight

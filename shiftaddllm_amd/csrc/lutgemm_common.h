@@ -64,6 +64,7 @@ constexpr int base_mode(int mode) { return is_staged(mode) ? mode - 4 : mode; }
 
 // compile-time input transform of a kernel instance
 constexpr int kXNone = 0, kXNorm = 1, kXGate = 2;
+constexpr int kXDynamic = 3;  // chained problems: one of the three, chosen at run time
 
 // Division by a run-time constant without a divide: n / d == umulhi((2 * n) >> shift,
 // magic), with the pair prepared on the host (kernels here start and end within a
@@ -154,6 +155,11 @@ struct Problem {
     const __half *next_w;   // [N]
     __half *next_in;        // [M][N]
     float *sumsq_out;       // [M][N / 32], zero before the launch
+    // Chained launches (lut_gemv_chain_kernel): a tag base of 0 means plain fp16 values; otherwise
+    // x / gate / out point at TAGGED rows, one 32-bit word per value = fp16 bits | tag << 16
+    // (see tagged_word below), x and gate are waited for, out is written with its tag.
+    int x_tag, gate_tag, out_tag;
+    int reserved2_;
 };
 static_assert(offsetof(Problem, by_group_words) == 64 && offsetof(Problem, gate) == 128 && offsetof(Problem, overwrite) == 192,
               "Problem: fields are grouped by cache line");
@@ -161,6 +167,30 @@ static_assert(offsetof(Problem, by_group_words) == 64 && offsetof(Problem, gate)
 struct Group {
     int count;
     Problem p[kMaxGroup];
+};
+
+// Tagged rows: how the problems of ONE launch hand activations to each other while all of them are
+// in flight.  A producer writes every finished value as one 32-bit word, fp16 bits | tag << 16,
+// with an agent-scope store (written through to memory, past the producer's L2); a consumer reads
+// the words it needs with agent-scope loads until all of them carry the tag it expects.  Value and
+// tag travel in one word, so no counter, no fence and no second round trip are needed: the
+// hand-over costs one store and one load latency.  The effective tag of base b in a launch whose
+// epoch word reads e is 1 + (b + e) % 65535: never 0, so zero-filled memory never matches, and
+// advancing the epoch between replays of a captured launch makes last replay's words stale.
+__host__ __device__ inline uint32_t effective_tag(int base, uint32_t epoch)
+{
+    return 1u + (uint32_t)(((unsigned long long)(uint32_t)base + epoch) % 65535ull);
+}
+
+struct ChainControl {
+    const uint32_t *epoch;   // device word added to every tag base (may be null: 0)
+    uint32_t *status;        // device word: bit 0 is set when a wait gave up
+    long long spin_ticks;    // bound of every wait, in ticks of the 100 MHz wall clock
+};
+
+struct Chain {
+    Group g;
+    ChainControl ctl;
 };
 
 __device__ __forceinline__ float half_bits_to_float(uint32_t bits16)

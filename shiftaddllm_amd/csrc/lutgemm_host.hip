@@ -138,6 +138,7 @@ struct Option {
 constexpr Option kOptions[LUTGEMM_OPTION_COUNT] = {
     {"LUTGEMM_TARGET_BLOCKS", 0}, {"LUTGEMM_FIRST_SHARE", 60}, {"LUTGEMM_MFMA_MIN_M", 3},
     {"LUTGEMM_MFMA_BLOCKS", 0},   {"LUTGEMM_PAIR_TABLES", 1},  {"LUTGEMM_SINGLE_ITEM", 1},
+    {"LUTGEMM_CHAIN_BLOCKS", 0},
 };
 std::atomic<int> g_option[LUTGEMM_OPTION_COUNT];
 std::once_flag g_option_once;
@@ -468,6 +469,56 @@ int run(int mode, const uint32_t *bW, const void *alpha, const void *qbias, cons
     return e == hipSuccess ? LUTGEMM_OK : hip_fail(e);
 }
 
+// Share a workgroup budget between look-up problems that run side by side so that the longest
+// range of every problem takes about the same time.  An item costs a table build plus look-ups in
+// proportion to its bit planes (0.45 + 0.13 * nb us measured), whatever the problem; the problems
+// end with their slowest workgroup, so the items per workgroup of problem i are floor(T / cost_i)
+// for the smallest T whose workgroups fit the budget.  (Sharing in proportion to the sign bytes
+// gave q,k,v of 2, 4 and 3 bits 5, 3 and 4 items per workgroup: 3.6, 2.9 and 3.4 us of work.)
+// With equal bit widths this is a share in proportion to the items, rounded down: a few
+// workgroups more than can be resident run as a second, mostly empty round, and fewer
+// workgroups with more items each are the better trade anyway (q,k,v of 4096x4096 as 3 x 64
+// workgroups of 4 items 5.31 us per GEMV of the four-launch block, as 3 x 86 of 3 items 5.54).
+// *most: the largest workgroup count of a problem (raised only); *any_split: some problem needs
+// accumulator words (set only).
+int share_workgroups(Problem *const *ps, int count, long budget, int *most, bool *any_split)
+{
+    long items[kMaxGroup];
+    double cost[kMaxGroup];
+    double lo = 0.0, hi = 0.0;
+    for (int i = 0; i < count; ++i) {
+        const Problem &p = *ps[i];
+        items[i] = (long)((p.N + kTileCols - 1) / kTileCols) * p.nsets;
+        cost[i] = 0.45 + 0.13 * p.nb;
+        const double all = (double)items[i] * cost[i];
+        if (all > hi) hi = all;
+    }
+    auto workgroups = [&](double t) {
+        long n = 0;
+        for (int i = 0; i < count; ++i) {
+            long ipw = (long)(t / cost[i]);
+            if (ipw < 1) return (long)1 << 40;
+            n += ((items[i] + ipw - 1) / ipw) * ps[i]->M;
+        }
+        return n;
+    };
+    for (int it = 0; it < 50; ++it) {
+        const double mid = 0.5 * (lo + hi);
+        if (workgroups(mid) <= budget) hi = mid; else lo = mid;
+    }
+    for (int i = 0; i < count; ++i) {
+        Problem &p = *ps[i];
+        long ipw = (long)(hi / cost[i]);
+        if (ipw < 1) ipw = 1;
+        const long want = ((items[i] + ipw - 1) / ipw) * p.M;
+        int rc = plan_lookup(p, 1, want);
+        if (rc != LUTGEMM_OK) return rc;
+        if (p.n_blocks > *most) *most = p.n_blocks;  // grid.x: the largest problem's workgroups
+        *any_split = *any_split || lookup_splits_k(p);
+    }
+    return LUTGEMM_OK;
+}
+
 // Up to kMaxGroup row-wise problems in one launch of the look-up kernel.  Problems
 // with enough rows for the matrix-core kernel (and no fused transform) are launched
 // on that path instead.
@@ -560,51 +611,13 @@ int run_group(int count, const lutgemm_fused_problem *problems, const Accum &acc
         }
         return LUTGEMM_OK;
     }
-    // Share the launch's workgroup budget so that the longest range of every problem takes about
-    // the same time.  An item costs a table build plus look-ups in proportion to its bit planes
-    // (0.45 + 0.13 * nb us measured), whatever the problem; the launch ends with its slowest
-    // workgroup, so the items per workgroup of problem i are floor(T / cost_i) for the smallest T
-    // whose workgroups fit the budget.  (Sharing in proportion to the sign bytes gave q,k,v of
-    // 2, 4 and 3 bits 5, 3 and 4 items per workgroup: 3.6, 2.9 and 3.4 us of work.)
-    // With equal bit widths this is a share in proportion to the items, rounded down: a few
-    // workgroups more than can be resident run as a second, mostly empty round, and fewer
-    // workgroups with more items each are the better trade anyway (q,k,v of 4096x4096 as 3 x 64
-    // workgroups of 4 items 5.31 us per GEMV of the four-launch block, as 3 x 86 of 3 items 5.54).
-    const long budget = (long)target_blocks(total_bytes);
-    long items[kMaxGroup];
-    double cost[kMaxGroup];
-    double lo = 0.0, hi = 0.0;
-    for (int i = 0; i < count; ++i) {
-        const Problem &p = g.p[i];
-        items[i] = (long)((p.N + kTileCols - 1) / kTileCols) * p.nsets;
-        cost[i] = 0.45 + 0.13 * p.nb;
-        const double all = (double)items[i] * cost[i];
-        if (all > hi) hi = all;
-    }
-    auto workgroups = [&](double t) {
-        long n = 0;
-        for (int i = 0; i < count; ++i) {
-            long ipw = (long)(t / cost[i]);
-            if (ipw < 1) return (long)1 << 40;
-            n += ((items[i] + ipw - 1) / ipw) * g.p[i].M;
-        }
-        return n;
-    };
-    for (int it = 0; it < 50; ++it) {
-        const double mid = 0.5 * (lo + hi);
-        if (workgroups(mid) <= budget) hi = mid; else lo = mid;
-    }
+    Problem *ps[kMaxGroup];
+    for (int i = 0; i < count; ++i) ps[i] = &g.p[i];
     int begin = 0;
     bool any_split = false;
-    for (int i = 0; i < count; ++i) {
-        Problem &p = g.p[i];
-        long ipw = (long)(hi / cost[i]);
-        if (ipw < 1) ipw = 1;
-        const long want = ((items[i] + ipw - 1) / ipw) * p.M;
-        int rc = plan_lookup(p, 1, want);
+    {
+        int rc = share_workgroups(ps, count, (long)target_blocks(total_bytes), &begin, &any_split);
         if (rc != LUTGEMM_OK) return rc;
-        if (p.n_blocks > begin) begin = p.n_blocks;  // grid.x: the largest problem's workgroups
-        any_split = any_split || lookup_splits_k(p);
     }
     if (any_split) {
         unsigned long long *base = nullptr;
@@ -618,6 +631,169 @@ int run_group(int count, const lutgemm_fused_problem *problems, const Accum &acc
     }
     const hipError_t e = count == 1 ? launch_gemv_fused(g.p[0], xform, acc.stream) : launch_gemv_group(g, xform, begin, acc.stream);
     return e == hipSuccess ? LUTGEMM_OK : hip_fail(e);
+}
+
+// Row-wise problems of ONE launch that hand activations to each other through tagged rows.
+// Problems are dispatched in the order given, so a problem that waits for a tag must come after
+// the problem of the call that writes it.  Problems that wait for the same set of producers run
+// side by side and share a workgroup budget (a "stage"); consecutive stages of at most 256
+// workgroups fit the chip together, so that a stage's operands stream while its producers compute.
+int chain_stage_blocks(long sign_bytes)
+{
+    const int v = option(LUTGEMM_OPTION_CHAIN_BLOCKS);
+    return v > 0 ? v : target_blocks(sign_bytes);
+}
+
+int run_chain(int count, const lutgemm_chain_problem *problems, const lutgemm_chain_control *ctl, const Accum &acc)
+{
+    if (!ctl || !ctl->status) return LUTGEMM_EINVAL;
+    if (!aligned(ctl->status, 4) || !aligned(ctl->epoch, 4)) return LUTGEMM_EALIGN;
+    Chain c{};
+    Group &g = c.g;
+    g.count = count;
+    size_t words = 0;
+    int depth[kMaxGroup];
+    unsigned direct[kMaxGroup], after[kMaxGroup], before_inputs[kMaxGroup];
+    for (int i = 0; i < count; ++i) {
+        const lutgemm_chain_problem &cq = problems[i];
+        const lutgemm_fused_problem &q = cq.p;
+        Problem &p = g.p[i];
+        int rc = fill_problem(p, kRowF16, q.bW, q.alpha_f16, nullptr, q.x_f16, q.out_f16, q.N, q.K, q.nb, q.num_groups, q.M);
+        if (rc != LUTGEMM_OK) return rc;
+        if (q.M > LUTGEMM_CHAIN_MAX_ROWS) return LUTGEMM_EUNSUP;   // one row per workgroup: the look-up kernel only
+        if (q.norm_weight_f16 && q.gate_f16) return LUTGEMM_EINVAL;
+        if (q.overwrite != 0 && q.overwrite != 1) return LUTGEMM_EINVAL;
+        if (q.norm_weight_f16 && !(q.norm_eps >= 0.0f)) return LUTGEMM_EINVAL;
+        if (!aligned(q.norm_weight_f16, 16) || !aligned(q.gate_f16, 16)) return LUTGEMM_EALIGN;
+        if (q.next_norm_weight_f16 || q.next_input_f16 || q.sumsq_out_f32 || q.sumsq_in_f32 || q.sumsq_in_slots)
+            return LUTGEMM_EUNSUP;   // the RMSNorm of a chained problem is formed from the (tagged) row itself
+        if (cq.x_tag < 0 || cq.x_tag > LUTGEMM_CHAIN_MAX_TAG || cq.gate_tag < 0 || cq.gate_tag > LUTGEMM_CHAIN_MAX_TAG ||
+            cq.out_tag < 0 || cq.out_tag > LUTGEMM_CHAIN_MAX_TAG)
+            return LUTGEMM_EINVAL;
+        if (cq.gate_tag && !q.gate_f16) return LUTGEMM_EINVAL;
+        // a thread holds its share of a norm row in two 16-byte registers sets: K <= 8192 when the row is tagged
+        if (q.norm_weight_f16 && cq.x_tag && q.K > 8 * 2 * kThreads) return LUTGEMM_EUNSUP;
+        p.norm_w = (const __half *)q.norm_weight_f16;
+        p.gate = (const __half *)q.gate_f16;
+        p.norm_eps = q.norm_eps;
+        p.overwrite = q.overwrite;
+        p.x_tag = cq.x_tag;
+        p.gate_tag = cq.gate_tag;
+        p.out_tag = cq.out_tag;
+        words += (size_t)q.M * q.N;
+        // which problems of the call this one waits for: the writers of the tags it reads
+        depth[i] = 0;
+        direct[i] = 0;
+        auto producer = [&](const void *row, int tag) -> int {
+            if (!tag) return LUTGEMM_OK;
+            for (int j = 0; j < count; ++j) {
+                if (problems[j].p.out_f16 != row || problems[j].out_tag != tag) continue;
+                if (j >= i) return LUTGEMM_EINVAL;   // dispatched after its consumer: the wait could starve it
+                direct[i] |= 1u << j;
+                if (depth[j] + 1 > depth[i]) depth[i] = depth[j] + 1;
+            }
+            return LUTGEMM_OK;   // (no writer in the call: the row comes from elsewhere, the wait is bounded)
+        };
+        rc = producer(q.x_f16, cq.x_tag);
+        if (rc != LUTGEMM_OK) return rc;
+        rc = producer(q.gate_f16, cq.gate_tag);
+        if (rc != LUTGEMM_OK) return rc;
+        if (i > 0 && depth[i] < depth[i - 1]) return LUTGEMM_EINVAL;   // stages in dispatch order
+        // everything this problem waits for, directly or not (after[i]), and through at least one
+        // other problem (before_inputs[i])
+        after[i] = direct[i];
+        before_inputs[i] = 0;
+        for (int j = 0; j < i; ++j)
+            if (direct[i] >> j & 1u) {
+                after[i] |= after[j];
+                before_inputs[i] |= after[j];
+            }
+    }
+    // What may overlap.  A problem writes an output only after contributions covering all of K
+    // have arrived, each of which has waited for its inputs: when problem i writes anything, every
+    // problem in after[i] has finished, and when a workgroup of i has its inputs, every problem in
+    // before_inputs[i] has.  So the same tagged row may be written by several problems of a call
+    // (a residual row that two GEMVs complete one after the other) and read in between, as long as
+    // the waits order them; plain rows may not be shared between a writer and anyone else.
+    for (int i = 0; i < count; ++i) {
+        const Problem &a = g.p[i];
+        const char *a0 = (const char *)a.out, *a1 = a0 + (size_t)a.M * a.N * (a.out_tag ? 4 : 2);
+        auto overlaps = [&](const void *ptr, size_t bytes) {
+            return ptr && a0 < (const char *)ptr + bytes && (const char *)ptr < a1;
+        };
+        for (int j = 0; j < count; ++j) {
+            if (i == j) continue;
+            const Problem &b = g.p[j];
+            if (j < i && overlaps(b.out, (size_t)b.M * b.N * (b.out_tag ? 4 : 2))) {
+                // an earlier writer of the same row: it must have finished before this one writes,
+                // and before this one reads the row when it accumulates into it
+                const bool same_row = a.out_tag && b.out_tag && a.out == b.out && a.out_tag != b.out_tag;
+                const unsigned need = a.overwrite ? after[i] : before_inputs[i];
+                if (!same_row || !(need >> j & 1u)) return LUTGEMM_EINVAL;
+            }
+            auto read_ok = [&](const __half *row, int tag, size_t bytes) {
+                if (!overlaps(row, bytes)) return true;
+                if (!(a.out_tag && tag && (const void *)row == (const void *)a.out)) return false;
+                if (tag == a.out_tag) return i < j;             // the hand-over itself
+                return (after[i] >> j & 1u) || (after[j] >> i & 1u);   // rewritten after the reader, or read after the writer
+            };
+            if (!read_ok(b.x, b.x_tag, (size_t)b.M * b.K * (b.x_tag ? 4 : 2))) return LUTGEMM_EINVAL;
+            if (!read_ok(b.gate, b.gate_tag, (size_t)b.M * b.K * (b.gate_tag ? 4 : 2))) return LUTGEMM_EINVAL;
+        }
+    }
+    // plan stage by stage
+    int begin = 0;
+    bool any_split = false;
+    for (int first = 0; first < count;) {
+        int last = first;
+        long bytes = 0;
+        Problem *ps[kMaxGroup];
+        while (last < count && depth[last] == depth[first]) {
+            ps[last - first] = &g.p[last];
+            bytes += (long)g.p[last].N * (g.p[last].K / 8) * g.p[last].nb * g.p[last].M;
+            ++last;
+        }
+        int rc = share_workgroups(ps, last - first, (long)chain_stage_blocks(bytes), &begin, &any_split);
+        if (rc != LUTGEMM_OK) return rc;
+        first = last;
+    }
+    for (int i = 0; i < count; ++i)   // a range's activations are fetched as one window
+        if (g.p[i].items_per_wg > kThreads / kTables) return LUTGEMM_EUNSUP;
+    if (any_split) {
+        unsigned long long *base = nullptr;
+        int rc = accum_words(acc, words, &base);
+        if (rc != LUTGEMM_OK) return rc;
+        size_t off = 0;
+        for (int i = 0; i < count; ++i) {
+            g.p[i].accum = base + off;
+            off += (size_t)g.p[i].M * g.p[i].N;
+        }
+    }
+    c.ctl.epoch = ctl->epoch;
+    c.ctl.status = ctl->status;
+    const unsigned us = ctl->spin_limit_us ? ctl->spin_limit_us : 100000u;
+    c.ctl.spin_ticks = (long long)us * 100;   // the wall clock ticks at 100 MHz
+    const hipError_t e = launch_gemv_chain(c, begin, acc.stream);
+    return e == hipSuccess ? LUTGEMM_OK : hip_fail(e);
+}
+
+// ---- tagged rows: conversions and the epoch word ---------------------------------------------
+__global__ void __launch_bounds__(256) tag_rows_kernel(uint32_t *dst, const unsigned short *src, size_t n, int tag,
+                                                       const uint32_t *epoch)
+{
+    const uint32_t t = effective_tag(tag, epoch ? *epoch : 0u) << 16;
+    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (size_t)gridDim.x * 256) dst[i] = t | src[i];
+}
+
+__global__ void __launch_bounds__(256) untag_rows_kernel(unsigned short *dst, const uint32_t *src, size_t n)
+{
+    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (size_t)gridDim.x * 256)
+        dst[i] = (unsigned short)src[i];
+}
+
+__global__ void advance_epoch_kernel(uint32_t *epoch, uint32_t by)
+{
+    if (threadIdx.x == 0 && blockIdx.x == 0) *epoch += by;
 }
 
 // ---- measurement kernels ------------------------------------------------------------
@@ -683,6 +859,8 @@ const char *lutgemm_strerror(int code)
     case LUTGEMM_ECAPTURE:
         return "the stream is being captured and its workspace would have to grow "
                "(call lutgemm_reserve_workspace before capturing)";
+    case LUTGEMM_ETIMEDOUT:
+        return "a problem of a chained launch gave up waiting for a tagged row (nothing wrote it within the limit)";
     case LUTGEMM_ETOOBIG:
         return "M * N exceeds LUTGEMM_NOALLOC_MAX_WORDS, the fixed buffer of the entry point that does not allocate";
     default: return "unknown lutgemm error";
@@ -750,6 +928,60 @@ int lutgemm_gemv_rowwise_f16_fused(int count, const lutgemm_fused_problem *probl
 {
     if (!problems || count < 1 || count > kMaxGroup) return LUTGEMM_EINVAL;
     return run_group(count, problems, Accum{(hipStream_t)stream_v});
+}
+
+int lutgemm_gemv_rowwise_f16_chain(int count, const lutgemm_chain_problem *problems,
+                                   const lutgemm_chain_control *control, void *stream_v)
+{
+    if (!problems || count < 1 || count > kMaxGroup) return LUTGEMM_EINVAL;
+    return run_chain(count, problems, control, Accum{(hipStream_t)stream_v});
+}
+
+int lutgemm_chain_tag_rows(void *dst_tagged, const void *src_f16, size_t count, int tag, const uint32_t *epoch,
+                           void *stream)
+{
+    if (!dst_tagged || !src_f16 || tag < 1 || tag > LUTGEMM_CHAIN_MAX_TAG) return LUTGEMM_EINVAL;
+    if (!aligned(dst_tagged, 4) || !aligned(src_f16, 2) || !aligned(epoch, 4)) return LUTGEMM_EALIGN;
+    if (count == 0) return LUTGEMM_OK;
+    size_t blocks = (count + 255) / 256;
+    if (blocks > 1024) blocks = 1024;
+    hipLaunchKernelGGL(tag_rows_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, (uint32_t *)dst_tagged,
+                       (const unsigned short *)src_f16, count, tag, epoch);
+    const hipError_t e = hipGetLastError();
+    return e == hipSuccess ? LUTGEMM_OK : hip_fail(e);
+}
+
+int lutgemm_chain_untag_rows(void *dst_f16, const void *src_tagged, size_t count, void *stream)
+{
+    if (!dst_f16 || !src_tagged) return LUTGEMM_EINVAL;
+    if (!aligned(dst_f16, 2) || !aligned(src_tagged, 4)) return LUTGEMM_EALIGN;
+    if (count == 0) return LUTGEMM_OK;
+    size_t blocks = (count + 255) / 256;
+    if (blocks > 1024) blocks = 1024;
+    hipLaunchKernelGGL(untag_rows_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream,
+                       (unsigned short *)dst_f16, (const uint32_t *)src_tagged, count);
+    const hipError_t e = hipGetLastError();
+    return e == hipSuccess ? LUTGEMM_OK : hip_fail(e);
+}
+
+int lutgemm_chain_advance_epoch(uint32_t *epoch, uint32_t by, void *stream)
+{
+    if (!epoch) return LUTGEMM_EINVAL;
+    if (!aligned(epoch, 4)) return LUTGEMM_EALIGN;
+    hipLaunchKernelGGL(advance_epoch_kernel, dim3(1), dim3(64), 0, (hipStream_t)stream, epoch, by);
+    const hipError_t e = hipGetLastError();
+    return e == hipSuccess ? LUTGEMM_OK : hip_fail(e);
+}
+
+int lutgemm_chain_status(const uint32_t *status, void *stream)
+{
+    if (!status) return LUTGEMM_EINVAL;
+    uint32_t v = 0;
+    hipError_t e = hipStreamSynchronize((hipStream_t)stream);
+    if (e != hipSuccess) return hip_fail(e);
+    e = hipMemcpy(&v, status, sizeof(v), hipMemcpyDeviceToHost);
+    if (e != hipSuccess) return hip_fail(e);
+    return v ? LUTGEMM_ETIMEDOUT : LUTGEMM_OK;
 }
 
 int lutgemm_gemv_uniform_f16(const uint32_t *bW, const void *alpha_f16, const void *qbias_f16,

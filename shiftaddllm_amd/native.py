@@ -24,6 +24,11 @@ C_ABI_SYMBOLS = (
     "lutgemm_gemv_rowwise_f16_noalloc",
     "lutgemm_gemv_rowwise_f16_grouped",
     "lutgemm_gemv_rowwise_f16_fused",
+    "lutgemm_gemv_rowwise_f16_chain",
+    "lutgemm_chain_tag_rows",
+    "lutgemm_chain_untag_rows",
+    "lutgemm_chain_advance_epoch",
+    "lutgemm_chain_status",
     "lutgemm_gemv_uniform_f16",
     "lutgemm_gemv_block_f16",
     "lutgemm_gemv_block_shift_u16",
@@ -45,7 +50,10 @@ C_ABI_SYMBOLS = (
 
 
 MAX_GROUP = 8
-OPTIONS = {"TARGET_BLOCKS": 0, "FIRST_SHARE": 1, "MFMA_MIN_M": 2, "MFMA_BLOCKS": 3, "PAIR_TABLES": 4, "SINGLE_ITEM": 5}
+OPTIONS = {"TARGET_BLOCKS": 0, "FIRST_SHARE": 1, "MFMA_MIN_M": 2, "MFMA_BLOCKS": 3, "PAIR_TABLES": 4, "SINGLE_ITEM": 5,
+           "CHAIN_BLOCKS": 6}
+CHAIN_MAX_ROWS = 4
+CHAIN_MAX_TAG = 65534
 NOALLOC_MAX_WORDS = 1 << 18
 
 
@@ -73,6 +81,16 @@ class FusedProblem(ctypes.Structure):
                 ("next_norm_weight_f16", ctypes.c_void_p), ("next_input_f16", ctypes.c_void_p),
                 ("sumsq_out_f32", ctypes.c_void_p), ("sumsq_in_f32", ctypes.c_void_p),
                 ("sumsq_in_slots", ctypes.c_int)]
+
+
+class ChainProblem(ctypes.Structure):
+    """struct lutgemm_chain_problem of include/lutgemm_gfx950.h."""
+    _fields_ = [("p", FusedProblem), ("x_tag", ctypes.c_int), ("gate_tag", ctypes.c_int), ("out_tag", ctypes.c_int)]
+
+
+class ChainControl(ctypes.Structure):
+    """struct lutgemm_chain_control of include/lutgemm_gfx950.h."""
+    _fields_ = [("epoch", ctypes.c_void_p), ("status", ctypes.c_void_p), ("spin_limit_us", ctypes.c_uint)]
 
 
 class NativeLibraryMissing(ImportError):
@@ -122,6 +140,16 @@ def cabi() -> ctypes.CDLL:
         lib.lutgemm_gemv_rowwise_f16_grouped.restype = ci
         lib.lutgemm_gemv_rowwise_f16_fused.argtypes = [ci, ctypes.POINTER(FusedProblem), vp]
         lib.lutgemm_gemv_rowwise_f16_fused.restype = ci
+        lib.lutgemm_gemv_rowwise_f16_chain.argtypes = [ci, ctypes.POINTER(ChainProblem), ctypes.POINTER(ChainControl), vp]
+        lib.lutgemm_gemv_rowwise_f16_chain.restype = ci
+        lib.lutgemm_chain_tag_rows.argtypes = [vp, vp, sz, ci, vp, vp]
+        lib.lutgemm_chain_tag_rows.restype = ci
+        lib.lutgemm_chain_untag_rows.argtypes = [vp, vp, sz, vp]
+        lib.lutgemm_chain_untag_rows.restype = ci
+        lib.lutgemm_chain_advance_epoch.argtypes = [vp, ctypes.c_uint, vp]
+        lib.lutgemm_chain_advance_epoch.restype = ci
+        lib.lutgemm_chain_status.argtypes = [vp, vp]
+        lib.lutgemm_chain_status.restype = ci
         lib.lutgemm_gemv_uniform_f16.argtypes = [vp, vp, vp, vp, vp, ci, ci, ci, ci, ci, vp]
         lib.lutgemm_gemv_block_f16.argtypes = [vp, vp, vp, vp, ci, ci, ci, ci, ci, vp]
         lib.lutgemm_gemv_block_shift_u16.argtypes = [vp, vp, vp, vp, ci, ci, ci, ci, ci, ci, vp]
