@@ -63,6 +63,9 @@ def parse_args():
                     help="N,K[,nb[,iters]]: only launch the floor kernels for this shape (empty launch; stream-read of the sign words) and exit")
     ap.add_argument("--profile-decode", type=int, default=0,
                     help="batch: only replay ten graph-captured decode steps of the 7B decoder (for rocprofv3 runs) and exit")
+    ap.add_argument("--profile-phases", type=str, default="",
+                    help="N,K[,nb[,iters]] or 'chain': run the shape (or one chained Llama-2-7B block) on the time-stamped "
+                         "build of the library and print where the time of a launch goes, then exit")
     ap.add_argument("--profile-copy", type=int, default=0,
                     help="bytes: only run the calibration copy kernel a few times (for rocprofv3 --pmc) and exit")
     return ap.parse_args()
@@ -162,6 +165,102 @@ def hf_opt_call_path(torch, dev):
     return res
 
 
+PHASES = ("entry", "operands_requested", "activations_arrived", "first_tables", "first_item", "all_items",
+          "handed_over", "exit")
+
+
+def profile_phases(torch, dev, spec, workload):
+    """Per-wave clock readings of the time-stamped library build (lutgemm_set_timestamp_buffer): for
+    every point the median and the latest wave, in microseconds since the first wave of the launch
+    started, per problem of the launch."""
+    import numpy as np
+    from shiftaddllm_amd import native
+    lib = native.cabi_timestamps()
+    stream = torch.cuda.Stream()
+    sp = ctypes.c_void_p(stream.cuda_stream)
+    slots = 4096 * 8 * 8
+    stamps = torch.zeros(slots, dtype=torch.int64, device=dev)
+
+    def check(rc):
+        if rc:
+            raise RuntimeError(lib.lutgemm_strerror(rc).decode())
+
+    def table(raw):
+        t = raw.reshape(-1, 8)
+        t = t[t[:, 0] != 0]
+        prob = (t[:, 0] >> 56) & 0xff
+        clock = (t & ((1 << 56) - 1)).astype(np.float64) * 0.01
+        clock = np.where(t != 0, clock, np.nan)          # (a point a wave did not pass)
+        t0 = np.nanmin(clock[:, 0])
+        out = {}
+        for y in sorted(set(prob.tolist())):
+            c = clock[prob == y] - t0
+            out[f"problem{y}"] = {"waves": int(c.shape[0]),
+                                  "median_us": {n: round(float(np.nanmedian(c[:, i])), 2) for i, n in enumerate(PHASES)},
+                                  "latest_us": {n: round(float(np.nanmax(c[:, i])), 2) for i, n in enumerate(PHASES)}}
+        return out
+
+    def run(launch, reps):
+        """launch(i) issues one launch on fresh operands; medians over the repetitions of every entry."""
+        tabs = []
+        for i in range(reps):
+            stamps.zero_()
+            torch.cuda.synchronize()
+            check(lib.lutgemm_set_timestamp_buffer(stamps.data_ptr(), slots))
+            with torch.cuda.stream(stream):
+                launch(i)
+            stream.synchronize()
+            tabs.append(table(stamps.cpu().numpy()))
+        check(lib.lutgemm_set_timestamp_buffer(None, 0))
+        tabs = tabs[1:] if len(tabs) > 1 else tabs        # the first launch also loads the code object
+        merged = {}
+        for key in tabs[0]:
+            merged[key] = {"waves": tabs[0][key]["waves"]}
+            for kind in ("median_us", "latest_us"):
+                merged[key][kind] = {n: round(float(np.median([t[key][kind][n] for t in tabs])), 2) for n in PHASES}
+        return merged
+
+    if spec != "chain":
+        parts = [int(v) for v in spec.split(",")]
+        N, K = parts[0], parts[1]
+        nb = parts[2] if len(parts) > 2 else NB
+        reps = parts[3] if len(parts) > 3 else 6
+        pool = [Gemv(torch, dev, N, K, nb, 300 + i) for i in range(reps)]
+        torch.cuda.synchronize()
+        res = run(lambda i: check(lib.lutgemm_gemv_rowwise_f16(*pool[i].args(), sp)), reps)
+        return {"shape": [N, K, nb], "launches": reps, "unit": "us since the first wave of the launch started",
+                "phases": res}
+    # one Llama-2-7B block, 3 bits, as ONE chained launch: q,k,v | o | gate,up | down
+    reps = 6
+    words = torch.zeros(2, dtype=torch.int32, device=dev)
+    ctl = native.ChainControl(words.data_ptr(), words.data_ptr() + 4, 0)
+    H, I = 4096, 11008
+    x0 = torch.randn((1, H), device=dev).half()
+    rows = {n: torch.zeros((1, w), dtype=torch.int32, device=dev) for n, w in
+            (("q", H), ("k", H), ("v", H), ("o", H), ("gate", I), ("up", I), ("down", H))}
+    blocks = []
+    for r in range(reps):
+        gs = [Gemv(torch, dev, N, K, NB, 500 + 10 * r + j) for j, (_, N, K) in enumerate(workload.LLAMA2_7B_LINEARS)]
+        fp = lambda g, x, out, gate=None: native.FusedProblem(
+            g.bW.data_ptr(), g.alpha.data_ptr(), x.data_ptr(), out.data_ptr(), g.N, g.K, g.nb, g.groups, 1, 1, None,
+            gate.data_ptr() if gate is not None else None, 1e-5)
+        cp = native.ChainProblem
+        arr = (cp * 7)(cp(fp(gs[0], x0, rows["q"]), 0, 0, 1), cp(fp(gs[1], x0, rows["k"]), 0, 0, 2),
+                       cp(fp(gs[2], x0, rows["v"]), 0, 0, 3), cp(fp(gs[3], rows["q"], rows["o"]), 1, 0, 4),
+                       cp(fp(gs[4], rows["o"], rows["gate"]), 4, 0, 5), cp(fp(gs[5], rows["o"], rows["up"]), 4, 0, 6),
+                       cp(fp(gs[6], rows["up"], rows["down"], gate=rows["gate"]), 6, 5, 7))
+        blocks.append((gs, arr))
+    torch.cuda.synchronize()
+
+    def launch(i):
+        check(lib.lutgemm_gemv_rowwise_f16_chain(7, blocks[i][1], ctypes.byref(ctl), sp))
+        check(lib.lutgemm_chain_advance_epoch(words.data_ptr(), 8, sp))
+    res = run(launch, reps)
+    return {"launch": "one Llama-2-7B block, 3 bits, chained: problems 0-2 q,k,v; 3 o (waits for q); 4,5 gate,up (wait for o); "
+                      "6 down (waits for gate and up)", "launches": reps,
+            "unit": "us since the first wave of the launch started", "phases": res}
+
+
 def main():
     args = parse_args()
     if args.gpus != 1:
@@ -241,6 +340,9 @@ def main():
         return statistics.median(ts)
 
     # ---- profiler helper modes --------------------------------------------
+    if args.profile_phases:
+        print(json.dumps(profile_phases(torch, dev, args.profile_phases, workload)))
+        return
     if args.profile_copy:
         nbytes = args.profile_copy // 16 * 16
         src = torch.empty(nbytes, dtype=torch.uint8, device=dev).random_(0, 255)
@@ -459,6 +561,68 @@ def main():
                         "us_per_gemv": round(dms * 1e3 / calls_per_step, 4),
                         "achieved_GBps": round(gbs, 1), "frac_hbm_peak": round(gbs / HBM_PEAK_GBS, 4),
                         "decode_tokens_per_s_linears_only": round(1e3 / dms, 1)}
+    # ---- the same block as ONE chained launch: q,k,v | o | gate,up | down hand their activations over
+    # inside the launch through tagged rows, so here the GEMVs really depend on each other (o reads q's
+    # output, gate and up read o's, down reads SiLU(gate) * up, the next block's q,k,v read down's)
+    if not args.plain_only:
+        words = torch.zeros(2, dtype=torch.int32, device=dev)
+        ctl = native.ChainControl(words.data_ptr(), words.data_ptr() + 4, 0)
+        H, I = 4096, 11008
+        x0 = torch.randn((1, H), device=dev).half()
+        i32 = dict(dtype=torch.int32, device=dev)
+        tq = [torch.zeros((1, H), **i32) for _ in range(3)]
+        to, tg, tu = torch.zeros((1, H), **i32), torch.zeros((1, I), **i32), torch.zeros((1, I), **i32)
+        tds = [torch.zeros((1, H), **i32) for _ in range(2)]        # down's output, alternating between blocks
+
+        def fp(g, x, out, gate=None):
+            return native.FusedProblem(g.bW.data_ptr(), g.alpha.data_ptr(), x.data_ptr(), out.data_ptr(), g.N, g.K, g.nb,
+                                       g.groups, 1, 1, None, gate.data_ptr() if gate is not None else None, 1e-5)
+        chained = []
+        cp = native.ChainProblem
+        for bi, b in enumerate(blocks):
+            t0, td, prev = 8 * bi, tds[bi % 2], tds[(bi - 1) % 2]
+            xin, xtag = (x0, 0) if bi == 0 else (prev, 8 * (bi - 1) + 7)
+            chained.append((cp * 7)(cp(fp(b[0], xin, tq[0]), xtag, 0, t0 + 1), cp(fp(b[1], xin, tq[1]), xtag, 0, t0 + 2),
+                                    cp(fp(b[2], xin, tq[2]), xtag, 0, t0 + 3), cp(fp(b[3], tq[0], to), t0 + 1, 0, t0 + 4),
+                                    cp(fp(b[4], to, tg), t0 + 4, 0, t0 + 5), cp(fp(b[5], to, tu), t0 + 4, 0, t0 + 6),
+                                    cp(fp(b[6], tu, td, gate=tg), t0 + 6, t0 + 5, t0 + 7)))
+
+        def seq_chained():
+            for arr in chained:
+                check(lib.lutgemm_gemv_rowwise_f16_chain(len(arr), arr, ctypes.byref(ctl), sp))
+            check(lib.lutgemm_chain_advance_epoch(words.data_ptr(), 8 * len(blocks), sp))
+        gr = capture(seq_chained)
+        _, dms = timed(seq_chained, gr, args.steps, args.warmup)
+        if lib.lutgemm_chain_status(words.data_ptr() + 4, sp):
+            raise SystemExit("a wait of the chained step gave up")
+        gbs = step_bytes / (dms * 1e-3) / 1e9
+        fused["chained_qkv_o_gateup_down"] = {
+            "launches_per_step": len(blocks) + 1, "device_ms_per_step": round(dms, 5),
+            "us_per_launch": round(dms * 1e3 / len(blocks), 3), "us_per_gemv": round(dms * 1e3 / calls_per_step, 4),
+            "achieved_GBps": round(gbs, 1), "frac_hbm_peak": round(gbs / HBM_PEAK_GBS, 4),
+            "decode_tokens_per_s_linears_only": round(1e3 / dms, 1)}
+        # parity of the chained block: its first and last GEMVs against separate launches on the same inputs
+        with torch.cuda.stream(stream):
+            check(lib.lutgemm_gemv_rowwise_f16_chain(7, chained[0], ctypes.byref(ctl), sp))
+            o_in, d_in, d_gate = (torch.empty((1, n), dtype=torch.float16, device=dev) for n in (H, I, I))
+            d_out = torch.empty((1, H), dtype=torch.float16, device=dev)
+            for dst, src in ((o_in, tq[0]), (d_in, tu), (d_gate, tg), (d_out, tds[0])):
+                check(lib.lutgemm_chain_untag_rows(dst.data_ptr(), src.data_ptr(), src.numel(), sp))
+            check(lib.lutgemm_chain_advance_epoch(words.data_ptr(), 8, sp))
+            ref_q = torch.zeros((1, H), dtype=torch.float16, device=dev)
+            ref_d = torch.zeros((1, H), dtype=torch.float16, device=dev)
+            b = blocks[0]
+            check(launch(vp(b[0].bW), vp(b[0].alpha), vp(x0), vp(ref_q), H, H, NB, b[0].groups, 1, sp))
+            arr1 = (native.FusedProblem * 1)(fp(b[6], d_in, ref_d, gate=d_gate))
+            check(lib.lutgemm_gemv_rowwise_f16_fused(1, arr1, sp))
+        stream.synchronize()
+        # (K is cut differently in a chained launch: agreement to fp16 rounding, not bit for bit)
+        parity["chained_first_gemv_rel_l2_vs_plain"] = oracle.error_metrics(o_in.float().cpu().numpy(), ref_q.float().cpu().numpy())[0]
+        parity["chained_last_gemv_rel_l2_vs_separate"] = oracle.error_metrics(d_out.float().cpu().numpy(), ref_d.float().cpu().numpy())[0]
+        if max(parity["chained_first_gemv_rel_l2_vs_plain"], parity["chained_last_gemv_rel_l2_vs_separate"]) > 2e-4:
+            raise SystemExit(f"chained launch disagrees with separate launches: {parity}")
+        del chained, tq, to, tg, tu, tds
+
     # parity of the fused path (outputs accumulate: clear, run once, compare with a plain call)
     if not args.plain_only:
         with torch.cuda.stream(stream):

@@ -267,7 +267,10 @@ int lutgemm_describe_plan(int format, int N, int K, int nb, int groups, int M, l
  *                   kernel, 0 = one fp32 table set per row
  *   SINGLE_ITEM   : 1 = launches whose ranges all hold one item take the kernel
  *                   instance that requests nothing beyond it, 0 = the general one
- *   CHAIN_BLOCKS  : workgroups per stage of a chained launch (0 = as TARGET_BLOCKS)
+ *   CHAIN_GRID    : workgroups of a chained launch (0 = as many as the device holds
+ *                   at once, which is also the upper limit)
+ *   CHAIN_BLOCKS  : ranges the problems of one stage of a chained launch are cut into
+ *                   (0 = one per workgroup of the launch)
  */
 #define LUTGEMM_OPTION_TARGET_BLOCKS 0
 #define LUTGEMM_OPTION_FIRST_SHARE 1
@@ -276,7 +279,8 @@ int lutgemm_describe_plan(int format, int N, int K, int nb, int groups, int M, l
 #define LUTGEMM_OPTION_PAIR_TABLES 4
 #define LUTGEMM_OPTION_SINGLE_ITEM 5
 #define LUTGEMM_OPTION_CHAIN_BLOCKS 6
-#define LUTGEMM_OPTION_COUNT 7
+#define LUTGEMM_OPTION_CHAIN_GRID 7
+#define LUTGEMM_OPTION_COUNT 8
 int lutgemm_set_option(int which, int value);
 int lutgemm_get_option(int which);
 
@@ -289,6 +293,23 @@ int lutgemm_get_option(int which);
  */
 int lutgemm_measure_stream_read(const void *src, size_t bytes, void *sink, void *stream);
 int lutgemm_measure_empty_launch(int workgroups, void *stream);
+
+/*
+ * Measurement helper of the time-stamped build of the library
+ * (liblutgemm_gfx950_ts.so, same sources compiled with -DLUTGEMM_TIMESTAMPS;
+ * the ordinary build returns LUTGEMM_EUNSUP).  After this call every wave of every
+ * look-up kernel launch writes LUTGEMM_STAMPS_PER_WAVE readings of the 100 MHz
+ * wall clock, taken at fixed points of the kernel (entry, first operands
+ * requested, activations arrived, first tables built, first item looked up, all
+ * items looked up, sums handed over, exit), into
+ *   readings[((workgroup of the grid) * 8 + wave) * LUTGEMM_STAMPS_PER_WAVE + point]
+ * (uint64, device memory, `count` readings of capacity; what does not fit is
+ * dropped; NULL switches the readings off).  The low 56 bits of a reading are the
+ * clock, the top byte is the workgroup's row of the grid: the problem of a grouped
+ * or chained launch, the row chunk of a lone one.  No counterpart in the reference.
+ */
+#define LUTGEMM_STAMPS_PER_WAVE 8
+int lutgemm_set_timestamp_buffer(void *readings, size_t count);
 
 /* Release the per-stream workspaces this library allocated on the current
  * device (optional; they otherwise live until the process ends).  HIP graphs

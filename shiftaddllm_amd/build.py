@@ -1,6 +1,8 @@
 """In-tree build of the two native pieces (no JIT cache, no install step).
 
   liblutgemm_gfx950.so          hipcc --offload-arch=gfx950, kernels + C ABI
+  liblutgemm_gfx950_ts.so       the same sources with -DLUTGEMM_TIMESTAMPS: the look-up
+                                kernels read the clock at fixed points (measurements only)
   lutgemm.cpython-*.so          g++, the `lutgemm` Python module (torch shim),
                                 linked against the library above via $ORIGIN
 
@@ -21,6 +23,7 @@ INCLUDE = os.path.join(REPO_DIR, "include")
 ROCM = os.environ.get("ROCM_PATH", "/opt/rocm")
 
 KERNEL_LIB = os.path.join(PKG_DIR, "liblutgemm_gfx950.so")
+KERNEL_LIB_TS = os.path.join(PKG_DIR, "liblutgemm_gfx950_ts.so")
 EXT_SUFFIX = sysconfig.get_config_var("EXT_SUFFIX") or ".so"
 TORCH_EXT = os.path.join(PKG_DIR, "lutgemm" + EXT_SUFFIX)
 
@@ -51,15 +54,17 @@ KERNEL_HEADERS = ("lutgemm_internal.h", "lutgemm_common.h", "lutgemm_launch.h", 
                   "lut_gemm_mfma_device.h")
 
 
-def build_kernel_library(force: bool = False) -> str:
-    """One object per source (only stale ones are recompiled, several at a time), linked into the library."""
+def build_kernel_library(force: bool = False, timestamps: bool = False) -> str:
+    """One object per source (only stale ones are recompiled, several at a time), linked into the library.
+    `timestamps`: the variant whose look-up kernels read the clock (-DLUTGEMM_TIMESTAMPS)."""
     from concurrent.futures import ThreadPoolExecutor
 
     hdrs = [os.path.join(INCLUDE, "lutgemm_gfx950.h")] + [os.path.join(CSRC, h) for h in KERNEL_HEADERS]
     hipcc = os.path.join(ROCM, "bin", "hipcc")
-    obj_dir = os.path.join(CSRC, "build")
+    obj_dir = os.path.join(CSRC, "build_ts" if timestamps else "build")
+    target = KERNEL_LIB_TS if timestamps else KERNEL_LIB
     os.makedirs(obj_dir, exist_ok=True)
-    flags = [f for f in HIPCC_FLAGS if f != "-shared"]
+    flags = [f for f in HIPCC_FLAGS if f != "-shared"] + (["-DLUTGEMM_TIMESTAMPS"] if timestamps else [])
     objs, stale = [], []
     for name in KERNEL_SOURCES:
         src = os.path.join(CSRC, name)
@@ -70,9 +75,9 @@ def build_kernel_library(force: bool = False) -> str:
     jobs = max(1, min(len(stale), int(os.environ.get("MAX_JOBS", "0")) or (os.cpu_count() or 4), 8))
     with ThreadPoolExecutor(max_workers=jobs) as pool:
         list(pool.map(_run, stale))
-    if stale or force or not _newer(KERNEL_LIB, *objs):
-        _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", KERNEL_LIB, *objs])
-    return KERNEL_LIB
+    if stale or force or not _newer(target, *objs):
+        _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", target, *objs])
+    return target
 
 
 def build_torch_extension(force: bool = False) -> str:
@@ -103,7 +108,7 @@ def build_torch_extension(force: bool = False) -> str:
 
 
 def build_all(force: bool = False):
-    return build_kernel_library(force), build_torch_extension(force)
+    return build_kernel_library(force), build_kernel_library(force, timestamps=True), build_torch_extension(force)
 
 
 if __name__ == "__main__":

@@ -229,6 +229,7 @@ struct ChainWait {
     uint32_t epoch;
     uint32_t *status;
     long long spin_ticks;
+    int unit, problem;   // of the launch (for the time-stamped build)
 };
 
 // Read NCH chunks of eight tagged words each (32 bytes at src[c]) until every word of every lane
@@ -238,6 +239,10 @@ struct ChainWait {
 // the values are meaningless.  The loads bypass the L2 (agent scope), which other workgroups'
 // stores are written through.  One asm statement holds the requests and their wait: the
 // compiler may place nothing that reads the destination registers in between.
+// A wave that finds a word without its tag does not read everything again at once (two thousand
+// waves re-reading kilobytes each microsecond would take a good part of the memory system from
+// the producers they wait for): it watches that one word, one four-byte request per round trip,
+// and reads everything again when the word has arrived.
 template <int NCH>
 __device__ __forceinline__ bool poll_tagged(const uint32_t *const (&src)[NCH], const uint32_t (&want)[NCH], u32x4 (&out)[NCH],
                                             const ChainWait &cw)
@@ -268,14 +273,17 @@ __device__ __forceinline__ bool poll_tagged(const uint32_t *const (&src)[NCH], c
                          "s_waitcnt vmcnt(0)"
                          : "=&v"(lo[0]), "=&v"(hi[0]), "=&v"(lo[1]), "=&v"(hi[1]), "=&v"(lo[2]), "=&v"(hi[2])
                          : "v"(src[0]), "v"(src[1]), "v"(src[2]) : "memory");
-        uint32_t bad = 0;
+        // the first word that does not carry its tag yet (-1: all of this lane's words do)
+        int missing = -1;
 #pragma unroll
-        for (int c = 0; c < NCH; ++c) {
+        for (int c = NCH - 1; c >= 0; --c) {
             const uint32_t w = want[c];
-            bad |= (lo[c].x ^ w) | (lo[c].y ^ w) | (lo[c].z ^ w) | (lo[c].w ^ w) | (hi[c].x ^ w) | (hi[c].y ^ w) |
-                   (hi[c].z ^ w) | (hi[c].w ^ w);
+            const uint32_t got8[8] = {lo[c].x, lo[c].y, lo[c].z, lo[c].w, hi[c].x, hi[c].y, hi[c].z, hi[c].w};
+#pragma unroll
+            for (int i = 7; i >= 0; --i) missing = ((got8[i] ^ w) & 0xffff0000u) ? 8 * c + i : missing;
         }
-        if (__builtin_amdgcn_ballot_w64((bad & 0xffff0000u) != 0) == 0) {
+        const unsigned long long late = __builtin_amdgcn_ballot_w64(missing >= 0);
+        if (late == 0) {
 #pragma unroll
             for (int c = 0; c < NCH; ++c) {
                 out[c].x = __builtin_amdgcn_perm(lo[c].y, lo[c].x, 0x05040100u);
@@ -285,12 +293,32 @@ __device__ __forceinline__ bool poll_tagged(const uint32_t *const (&src)[NCH], c
             }
             return true;
         }
-        if (__hip_atomic_load(cw.status, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u) return false;
-        if (wall_clock64() - t0 > cw.spin_ticks) {
-            if ((threadIdx.x & 63) == 0) __hip_atomic_fetch_or(cw.status, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            return false;
+        // watch the missing word of the first lane that has one (the same address in every lane:
+        // one request)
+        const int first = (int)__builtin_ctzll(late);
+        const int which = __builtin_amdgcn_readlane(missing, first);
+        const uint32_t *chunk = src[0];
+        uint32_t watch_want = want[0];
+#pragma unroll
+        for (int c = 1; c < NCH; ++c)
+            if ((which >> 3) == c) {
+                chunk = src[c];
+                watch_want = want[c];
+            }
+        const unsigned long long addr = (unsigned long long)(chunk + (which & 7));
+        const uint32_t *watch = (const uint32_t *)(((unsigned long long)(uint32_t)__builtin_amdgcn_readlane((int)(addr >> 32), first) << 32) |
+                                                   (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)addr, first));
+        watch_want = (uint32_t)__builtin_amdgcn_readlane((int)watch_want, first);
+        for (;;) {
+            const uint32_t v = __hip_atomic_load(watch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if (((v ^ watch_want) & 0xffff0000u) == 0) break;
+            if (__hip_atomic_load(cw.status, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u) return false;
+            if (wall_clock64() - t0 > cw.spin_ticks) {
+                if ((threadIdx.x & 63) == 0) __hip_atomic_fetch_or(cw.status, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                return false;
+            }
+            __builtin_amdgcn_s_sleep(4);
         }
-        __builtin_amdgcn_s_sleep(2);
     }
 }
 
@@ -647,8 +675,15 @@ __device__ __forceinline__ float reduce_scatter_kw(const float (&acc)[4], int kw
 //      requested at once; the activations are waited for, tag by tag, behind them.
 template <int NB, int MODE, int MROWS, int XF = kXNone, bool EXTRA = false, int ALONE = MROWS == 1 && !is_block(MODE),
           bool PAIR = false, bool DEP = false>
-__device__ __forceinline__ void gemv_range(const Problem &p, int range, int mchunk, float *lut, const ChainWait *cw = nullptr)
+__device__ __forceinline__ bool gemv_range(const Problem &p, int range, int mchunk, float *lut, const ChainWait *cw = nullptr)
 {
+    // Returns false when a chained problem gave up waiting for its inputs (nothing was written).
+    [[maybe_unused]] auto stamp = [&](const Problem &pp, int point) {
+        if constexpr (DEP)
+            lutgemm::stamp(pp, point, cw->unit, cw->problem);
+        else
+            lutgemm::stamp(pp, point, (long long)blockIdx.y * gridDim.x + blockIdx.x, (int)blockIdx.y);
+    };
     static_assert(!PAIR || (MROWS % 2 == 0 && (MODE == kRowF16 || MODE == kUniformF16)), "pair tables: even row count, per-column alphas");
     static_assert(!(EXTRA || XF == kXNorm) || !is_staged(MODE), "the per-wave sums live in the alpha staging area");
     static_assert(!DEP || (MROWS == 1 && MODE == kRowF16 && !EXTRA && !PAIR), "chained launches: one row per workgroup, row-wise alphas");
@@ -658,6 +693,7 @@ __device__ __forceinline__ void gemv_range(const Problem &p, int range, int mchu
     // eight instances of this function on, it emits an empty kernel)
     [[maybe_unused]] const int xf = XF != kXDynamic ? XF : p.norm_w ? kXNorm : p.gate ? kXGate : kXNone;
     constexpr bool kMayNorm = XF == kXNorm || XF == kXDynamic;
+    stamp(p, kStampEntry);
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = tid >> 6;
@@ -714,9 +750,11 @@ __device__ __forceinline__ void gemv_range(const Problem &p, int range, int mchu
     constexpr int kSlots = kWindowSlots / MROWS;  // items per window
     const int set0 = set, n_items = rem;
     float *window = stage + kStageDwords;
-    // (a chained problem requests its activations later, behind the first two items' operands)
+    // (a chained problem that waits for a tag requests its activations later, behind the first
+    // item's sign words)
     WindowChunk w0;
     if constexpr (!DEP) w0 = fetch_window<MROWS, XF>(p, m0, set0, 0, n_items, tid);
+    [[maybe_unused]] const bool chain_waits = DEP && (p.x_tag != 0 || p.gate_tag != 0);
     constexpr bool kDirectFirst = XF == kXNone && !PAIR && !DEP;
     // Without an input transform the tables of the first item (row 0) are built straight
     // from a second request for this thread's own chunk, so that nothing but that chunk
@@ -804,6 +842,8 @@ __device__ __forceinline__ void gemv_range(const Problem &p, int range, int mchu
             return ok;
         }
     };
+    if constexpr (DEP)
+        if (!chain_waits) (void)chain_inputs();   // plain rows: requested first, like a lone problem's
     // split RMSNorm, consuming side: this thread's share of the rows' sums of squares
     float slot_sum[MROWS];
 #pragma unroll
@@ -894,6 +934,7 @@ __device__ __forceinline__ void gemv_range(const Problem &p, int range, int mchu
             }
         }
         store_window<MROWS, XF>(w0, window, tid, xf);
+        stamp(p, kStampInputs);
         // (without a transform the first build does not read the window, and the barrier
         // that follows that build publishes the window as well)
         if constexpr (!kDirectFirst) __syncthreads();
@@ -1040,6 +1081,7 @@ __device__ __forceinline__ void gemv_range(const Problem &p, int range, int mchu
             if (r == 0) stage_alpha<NB, MODE>(ops, stage, abuf, tid);
             __syncthreads();
             if (r == 0) {
+                if (rel == 0) stamp(p, kStampTables);
                 __builtin_amdgcn_sched_barrier(0);
                 after_first_barrier();
                 __builtin_amdgcn_sched_barrier(0);
@@ -1052,11 +1094,14 @@ __device__ __forceinline__ void gemv_range(const Problem &p, int range, int mchu
             lane_off ^= kFlip;
         }
         abuf ^= 1;
+        if (rel == 0) stamp(p, kStampFirstItem);
         ++rel;
+        if (last) stamp(p, kStampItems);
         if (last || nt != tile) {
             flush_tile(tile);
             if (!last) fetch_out(nt);
         }
+        if (last) stamp(p, kStampHandedOver);
         tile = nt;
         set = ns;
     };
@@ -1088,40 +1133,7 @@ __device__ __forceinline__ void gemv_range(const Problem &p, int range, int mchu
     int ld_tile = tile, ld_set = set;  // next item to request
     const int pairs = (n_items + 1) / 2;
     auto no_hook = []() {};
-    if constexpr (DEP) {
-        // Chained problem: the first two items' operands are requested at once (the workgroup
-        // may have to wait for its activations anyway, and whatever arrives meanwhile is off
-        // the path that starts when they do); then the activations, tag by tag.
-        load_item<NB, MODE>(opA, p, ld_tile, ld_set, true, kw, q, lane_col, tid);
-        advance(ld_tile, ld_set);
-        load_item<NB, MODE>(opB, p, ld_tile, ld_set, 1 < n_items, kw, q, lane_col, tid);
-        advance(ld_tile, ld_set);
-        __builtin_amdgcn_sched_barrier(0);
-        late_setup();
-        out_tagw = effective_tag(p.out_tag, cw->epoch) << 16;
-        const bool ok = chain_inputs();
-        // every wave leaves its verdict where the others read it behind first_window's barrier:
-        // a workgroup goes on or gives up as a whole
-        if (lane == 0) stage[64 + wave] = ok ? 0.0f : 1.0f;
-        fetch_out(tile);
-        first_window();
-        float gave_up = 0.0f;
-#pragma unroll
-        for (int w = 0; w < kWaves; ++w) gave_up += stage[64 + w];
-        if (gave_up != 0.0f) return;
-        item_step(opA, n_items == 1, no_hook);
-#pragma clang loop unroll(disable)
-        for (int j = 1; j < pairs; ++j) {
-            load_item<NB, MODE>(opA, p, ld_tile, ld_set, true, kw, q, lane_col, tid);
-            advance(ld_tile, ld_set);
-            item_step(opB, false, no_hook);
-            const bool has_b = 2 * j + 1 < n_items;
-            load_item<NB, MODE>(opB, p, ld_tile, ld_set, has_b, kw, q, lane_col, tid);
-            advance(ld_tile, ld_set);
-            item_step(opA, !has_b, no_hook);
-        }
-        if ((n_items & 1) == 0) item_step(opB, true, no_hook);
-    } else if constexpr (ALONE == 2) {
+    if constexpr (ALONE == 2) {
         // One item per range, known at launch: nothing is requested for a second item.  In the
         // general form below a range that ends requests a dummy in place of the item that
         // does not exist (so that every wait can count its loads), and those six to eight
@@ -1129,6 +1141,7 @@ __device__ __forceinline__ void gemv_range(const Problem &p, int range, int mchu
         // 4096x4096 3-bit 5.1 -> 4.8 us, 4-bit 6.1 -> 5.3, 3072x768 3-bit 4.4 -> 3.8.
         load_item<NB, MODE, 1>(opA, p, ld_tile, ld_set, true, kw, q, lane_col, tid);
         __builtin_amdgcn_sched_barrier(0);
+        stamp(p, kStampRequested);
         late_setup();
         first_window();
         load_item<NB, MODE, 2>(opA, p, ld_tile, ld_set, true, kw, q, lane_col, tid);
@@ -1136,8 +1149,25 @@ __device__ __forceinline__ void gemv_range(const Problem &p, int range, int mchu
     } else if constexpr (ALONE == 1) {
         load_item<NB, MODE, 1>(opA, p, ld_tile, ld_set, true, kw, q, lane_col, tid);
         __builtin_amdgcn_sched_barrier(0);
+        stamp(p, kStampRequested);
         late_setup();
+        if constexpr (DEP) {
+            // Chained problem that waits: its activations are read, tag by tag, behind the first
+            // item's sign words (which depend on nothing and stream meanwhile).  Every wave leaves
+            // its verdict where the others read it behind first_window's barrier: a workgroup
+            // goes on or gives up as a whole.
+            out_tagw = effective_tag(p.out_tag, cw->epoch) << 16;
+            bool ok = true;
+            if (chain_waits) ok = chain_inputs();
+            if (lane == 0) stage[64 + wave] = ok ? 0.0f : 1.0f;
+        }
         first_window();
+        if constexpr (DEP) {
+            float gave_up = 0.0f;
+#pragma unroll
+            for (int w = 0; w < kWaves; ++w) gave_up += stage[64 + w];
+            if (gave_up != 0.0f) return false;
+        }
         load_item<NB, MODE, 2>(opA, p, ld_tile, ld_set, true, kw, q, lane_col, tid);
         advance(ld_tile, ld_set);
         item_step(opA, n_items == 1, [&]() {
@@ -1173,6 +1203,7 @@ __device__ __forceinline__ void gemv_range(const Problem &p, int range, int mchu
             load_item<NB, MODE>(opB, p, ld_tile, ld_set, has_b, kw, q, lane_col, tid);
             advance(ld_tile, ld_set);
             if (first) {
+                stamp(p, kStampRequested);
                 late_setup();
                 fetch_out(tile);
                 first_window();
@@ -1181,6 +1212,8 @@ __device__ __forceinline__ void gemv_range(const Problem &p, int range, int mchu
         }
         if ((n_items & 1) == 0) item_step(opB, true, no_hook);
     }
+    stamp(p, kStampExit);
+    return true;
 }
 
 // Flat workgroup index (relative to the problem) -> (range, row chunk), for launches

@@ -160,6 +160,13 @@ struct Problem {
     // (see tagged_word below), x and gate are waited for, out is written with its tag.
     int x_tag, gate_tag, out_tag;
     int reserved2_;
+#ifdef LUTGEMM_TIMESTAMPS
+    // Build with per-wave time stamps (the library variant bench.py --profile-phases loads):
+    // kStampsPerWave readings of the 100 MHz wall clock per wave, at fixed points of the
+    // look-up kernel, into stamps[((workgroup of the grid) * kWaves + wave) * kStampsPerWave + point].
+    unsigned long long *stamps;
+    long long stamp_slots;   // capacity in readings
+#endif
 };
 static_assert(offsetof(Problem, by_group_words) == 64 && offsetof(Problem, gate) == 128 && offsetof(Problem, overwrite) == 192,
               "Problem: fields are grouped by cache line");
@@ -188,10 +195,46 @@ struct ChainControl {
     long long spin_ticks;    // bound of every wait, in ticks of the 100 MHz wall clock
 };
 
+// A chained launch is persistent: `grid` workgroups, all resident at once, walk the launch's
+// units (a unit = one workgroup's range of one problem, numbered problem by problem) in steps of
+// `grid`.  unit_start[y] is the first unit of problem y, unit_start[count] the number of units.
 struct Chain {
     Group g;
     ChainControl ctl;
+    int unit_start[kMaxGroup + 1];
+    int reserved_;
 };
+
+// Points of the look-up kernel at which the time-stamped build reads the clock.
+constexpr int kStampsPerWave = 8;
+enum StampPoint : int {
+    kStampEntry = 0,       // first instruction of the workgroup
+    kStampRequested = 1,   // the first operands (sign words, alphas) have been requested
+    kStampInputs = 2,      // the activations have arrived (and, in a chained launch, carry their tags)
+    kStampTables = 3,      // first tables built, first barrier passed
+    kStampFirstItem = 4,   // first item looked up
+    kStampItems = 5,       // all items looked up (the last hand-over is next)
+    kStampHandedOver = 6,  // sums handed over: atomics returned, outputs written
+    kStampExit = 7,
+};
+
+// `wg`: the workgroup's slot among the readings (its place in the grid, or the unit it works on in a
+// persistent launch); `row`: its row of the grid or the problem it works on.
+__device__ __forceinline__ void stamp(const Problem &p, int point, long long wg, int row)
+{
+#ifdef LUTGEMM_TIMESTAMPS
+    if (p.stamps && (threadIdx.x & 63) == 0) {
+        const long long at = (wg * kWaves + (threadIdx.x >> 6)) * kStampsPerWave + point;
+        // (the clock needs 56 bits in 22 years: the top byte names the row)
+        if (at < p.stamp_slots) p.stamps[at] = (wall_clock64() & ((1ull << 56) - 1)) | ((unsigned long long)row << 56);
+    }
+#else
+    (void)p;
+    (void)point;
+    (void)wg;
+    (void)row;
+#endif
+}
 
 __device__ __forceinline__ float half_bits_to_float(uint32_t bits16)
 {

@@ -26,6 +26,10 @@ constexpr int kMaxDevices = 64;
 
 thread_local int g_last_hip_error = 0;
 
+// time-stamped build only: where the kernels leave their clock readings
+std::atomic<unsigned long long *> g_stamps{nullptr};
+std::atomic<long long> g_stamp_slots{0};
+
 int hip_fail(hipError_t e)
 {
     g_last_hip_error = (int)e;
@@ -138,7 +142,7 @@ struct Option {
 constexpr Option kOptions[LUTGEMM_OPTION_COUNT] = {
     {"LUTGEMM_TARGET_BLOCKS", 0}, {"LUTGEMM_FIRST_SHARE", 60}, {"LUTGEMM_MFMA_MIN_M", 3},
     {"LUTGEMM_MFMA_BLOCKS", 0},   {"LUTGEMM_PAIR_TABLES", 1},  {"LUTGEMM_SINGLE_ITEM", 1},
-    {"LUTGEMM_CHAIN_BLOCKS", 0},
+    {"LUTGEMM_CHAIN_BLOCKS", 0}, {"LUTGEMM_CHAIN_GRID", 0},
 };
 std::atomic<int> g_option[LUTGEMM_OPTION_COUNT];
 std::once_flag g_option_once;
@@ -277,6 +281,10 @@ int fill_problem(Problem &p, int mode, const uint32_t *bW, const void *alpha, co
         if (p.rows_per_group % 4 != 0) return LUTGEMM_EINVAL;
     }
     p.by_group_words = make_divisor(p.group_words);
+#ifdef LUTGEMM_TIMESTAMPS
+    p.stamps = g_stamps.load();
+    p.stamp_slots = g_stamp_slots.load();
+#endif
     // the multiply-high divisions of the kernels are exact within these bounds
     const unsigned long long tiles = (unsigned long long)(N + kTileCols - 1) / kTileCols;
     if (2ull * p.kwords * p.group_words >= (1ull << 32)) return LUTGEMM_EUNSUP;
@@ -634,14 +642,21 @@ int run_group(int count, const lutgemm_fused_problem *problems, const Accum &acc
 }
 
 // Row-wise problems of ONE launch that hand activations to each other through tagged rows.
-// Problems are dispatched in the order given, so a problem that waits for a tag must come after
+// The launch's units (one workgroup's range of one problem) are numbered in the order the
+// problems are given and taken in that order, so a problem that waits for a tag must come after
 // the problem of the call that writes it.  Problems that wait for the same set of producers run
-// side by side and share a workgroup budget (a "stage"); consecutive stages of at most 256
-// workgroups fit the chip together, so that a stage's operands stream while its producers compute.
-int chain_stage_blocks(long sign_bytes)
+// side by side and share a workgroup budget (a "stage").
+// Workgroups of a chained launch: all of them must be resident at once (a unit may wait for a
+// unit of another workgroup), so at most what the device holds of this kernel.
+int chain_grid(int *out)
 {
-    const int v = option(LUTGEMM_OPTION_CHAIN_BLOCKS);
-    return v > 0 ? v : target_blocks(sign_bytes);
+    int resident = 0;
+    const hipError_t e = chain_resident_workgroups(&resident);
+    if (e != hipSuccess) return hip_fail(e);
+    if (resident < 1) return LUTGEMM_EUNSUP;
+    const int v = option(LUTGEMM_OPTION_CHAIN_GRID);
+    *out = v > 0 && v < resident ? v : resident;
+    return LUTGEMM_OK;
 }
 
 int run_chain(int count, const lutgemm_chain_problem *problems, const lutgemm_chain_control *ctl, const Accum &acc)
@@ -741,7 +756,14 @@ int run_chain(int count, const lutgemm_chain_problem *problems, const lutgemm_ch
             if (!read_ok(b.gate, b.gate_tag, (size_t)b.M * b.K * (b.gate_tag ? 4 : 2))) return LUTGEMM_EINVAL;
         }
     }
-    // plan stage by stage
+    // Plan stage by stage: the problems of a stage share one round of the grid (every workgroup
+    // takes one unit of the stage) unless LUTGEMM_OPTION_CHAIN_BLOCKS says otherwise.
+    int grid = 0;
+    {
+        int rc = chain_grid(&grid);
+        if (rc != LUTGEMM_OK) return rc;
+    }
+    const int stage_blocks = option(LUTGEMM_OPTION_CHAIN_BLOCKS) > 0 ? option(LUTGEMM_OPTION_CHAIN_BLOCKS) : grid;
     int begin = 0;
     bool any_split = false;
     for (int first = 0; first < count;) {
@@ -753,7 +775,7 @@ int run_chain(int count, const lutgemm_chain_problem *problems, const lutgemm_ch
             bytes += (long)g.p[last].N * (g.p[last].K / 8) * g.p[last].nb * g.p[last].M;
             ++last;
         }
-        int rc = share_workgroups(ps, last - first, (long)chain_stage_blocks(bytes), &begin, &any_split);
+        int rc = share_workgroups(ps, last - first, (long)stage_blocks, &begin, &any_split);
         if (rc != LUTGEMM_OK) return rc;
         first = last;
     }
@@ -773,7 +795,11 @@ int run_chain(int count, const lutgemm_chain_problem *problems, const lutgemm_ch
     c.ctl.status = ctl->status;
     const unsigned us = ctl->spin_limit_us ? ctl->spin_limit_us : 100000u;
     c.ctl.spin_ticks = (long long)us * 100;   // the wall clock ticks at 100 MHz
-    const hipError_t e = launch_gemv_chain(c, begin, acc.stream);
+    c.unit_start[0] = 0;
+    for (int i = 0; i < count; ++i) c.unit_start[i + 1] = c.unit_start[i] + g.p[i].n_blocks;
+    for (int i = count; i < kMaxGroup; ++i) c.unit_start[i + 1] = c.unit_start[count];
+    const int total_units = c.unit_start[count];
+    const hipError_t e = launch_gemv_chain(c, total_units < grid ? total_units : grid, acc.stream);
     return e == hipSuccess ? LUTGEMM_OK : hip_fail(e);
 }
 
@@ -868,6 +894,20 @@ const char *lutgemm_strerror(int code)
 }
 
 int lutgemm_last_hip_error(void) { return g_last_hip_error; }
+
+int lutgemm_set_timestamp_buffer(void *readings, size_t count)
+{
+#ifdef LUTGEMM_TIMESTAMPS
+    if (!aligned(readings, 8) || (count > 0 && !readings)) return LUTGEMM_EINVAL;
+    g_stamps.store((unsigned long long *)readings);
+    g_stamp_slots.store((long long)count);
+    return LUTGEMM_OK;
+#else
+    (void)readings;
+    (void)count;
+    return LUTGEMM_EUNSUP;   // this build of the library reads no clocks
+#endif
+}
 
 int lutgemm_set_option(int which, int value)
 {

@@ -19,8 +19,10 @@ hipError_t launch_gemv_block_staged(const Problem &p, int mode, int mrows, hipSt
 hipError_t launch_gemv_fused(const Problem &p, int xform, hipStream_t stream);
 // look-up kernel, several row-wise problems; grid = (blocks of the largest problem, problems)
 hipError_t launch_gemv_group(const Group &g, int xform, int blocks, hipStream_t stream);
-// look-up kernel, chained row-wise problems; grid = (blocks of the largest problem, problems)
+// look-up kernel, chained row-wise problems; persistent grid of `blocks` workgroups
 hipError_t launch_gemv_chain(const Chain &c, int blocks, hipStream_t stream);
+// workgroups of that kernel the current device holds at once (looked up once per device)
+hipError_t chain_resident_workgroups(int *count);
 // matrix-core kernel; mt = 1 (16-row tiles) or 2 (32-row tiles)
 hipError_t launch_mfma(const Problem &p, int mt, hipStream_t stream);
 hipError_t launch_mfma_fused(const Problem &p, int mt, hipStream_t stream);  // one problem with fused extras

@@ -98,11 +98,15 @@ class LutDecoder(nn.Module):
 
     def __init__(self, cfg: DecoderConfig, quant_config: dict | None = None, batch: int = 1, seed: int = 0,
                  device="cuda:0", default_bits: int = 3, fuse_launches: bool = True,
-                 module_prefix: str = "model.layers", glue: str = "hip"):
+                 module_prefix: str = "model.layers", glue: str = "hip", chain: bool = False):
         super().__init__()
         if glue not in ("hip", "torch"):
             raise ValueError(f"glue must be 'hip' or 'torch', got {glue!r}")
         self.cfg, self.batch, self.fuse, self.glue = cfg, batch, fuse_launches, glue
+        # o_proj, gate/up, down_proj and the next block's q,k,v as ONE chained launch per block (tagged
+        # rows hand the activations over inside the launch): two launches per block with the attention
+        # kernel.  One or two sequences (the chained launch runs on the look-up kernel), hidden <= 8192.
+        self.chain = bool(chain) and fuse_launches and glue == "hip" and batch <= 2 and cfg.hidden <= 8192
         # One or two sequences: RMSNorm inside the q,k,v and gate,up GEMVs (every workgroup re-reads
         # the row to form its RMS and scales its finished sums; the look-up kernel only).  Measured
         # against the split below on the 7B decoder at one sequence: 1.535 vs 1.572 ms per token.
@@ -149,8 +153,22 @@ class LutDecoder(nn.Module):
         self.register_buffer("act", torch.zeros((batch, I), **f16), persistent=False)
         self.register_buffer("sumsq", torch.zeros((2 * cfg.layers, batch, max(cfg.hidden // 32, 1)),
                                                   dtype=torch.float32, device=dev), persistent=False)
+        if self.chain:
+            i32 = dict(dtype=torch.int32, device=dev)
+            self.register_buffer("x_tagged", torch.zeros((batch, cfg.hidden), **i32), persistent=False)
+            self.register_buffer("gate_tagged", torch.zeros((batch, I), **i32), persistent=False)
+            self.register_buffer("up_tagged", torch.zeros((batch, I), **i32), persistent=False)
+            self.register_buffer("chain_words", torch.zeros((2,), **i32), persistent=False)   # epoch, status
         self._graph = None
         self._stream = None
+
+    def chain_status(self):
+        """0, or -8 when a wait inside a chained launch gave up since the status word was last cleared
+        (synchronises the current stream)."""
+        if not self.chain:
+            return 0
+        return native.cabi().lutgemm_chain_status(self.chain_words.data_ptr() + 4,
+                                                  ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
 
     # ---- linear layers -----------------------------------------------------------------
     def _fused(self, lins, x):
@@ -220,7 +238,60 @@ class LutDecoder(nn.Module):
         if rc:
             raise RuntimeError(lib.lutgemm_strerror(rc).decode())
 
+    def _step_chained(self):
+        """glue="hip" with chain=True: per block the attention kernel and ONE chained launch."""
+        cfg, B = self.cfg, self.batch
+        hd, H, KV, I = cfg.head_dim, cfg.heads, cfg.kv_heads, cfg.intermediate
+        lib = native.cabi()
+        sp = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+        def check(rc):
+            if rc:
+                raise RuntimeError(lib.lutgemm_strerror(rc).decode())
+
+        nq, nkv = B * H * hd, B * KV * hd
+        q, k, v = self.qkv[:nq], self.qkv[nq:nq + nkv], self.qkv[nq + nkv:]
+        x, h, xt, gt, ut = self.x_res, self.h_norm, self.x_tagged, self.gate_tagged, self.up_tagged
+        epoch = self.chain_words.data_ptr()
+        ctl = native.ChainControl(epoch, epoch + 4, 0)
+
+        def problem(lin, src, dst, x_tag=0, gate_tag=0, out_tag=0, norm=None, gate=None, overwrite=False):
+            return native.ChainProblem(
+                native.FusedProblem(lin.binaryWeight.data_ptr(), lin.alpha.data_ptr(), src.data_ptr(), dst.data_ptr(), lin.N,
+                                    lin.K, lin.wbit, lin.num_groups, B, int(overwrite),
+                                    norm.data_ptr() if norm is not None else None,
+                                    gate.data_ptr() if gate is not None else None, cfg.rms_eps),
+                x_tag, gate_tag, out_tag)
+
+        torch.index_select(self.embed, 0, self.ids, out=x)
+        check(lib.lutgemm_chain_tag_rows(xt.data_ptr(), x.data_ptr(), x.numel(), 255, epoch, sp))
+        first = self.blocks[0]
+        self._fused_gemv([first.q_proj, first.k_proj, first.v_proj], x, [q, k, v], sp, norm=first.input_norm, overwrite=True)
+        for li, blk in enumerate(self.blocks):
+            check(lib.lutgemm_decode_attention_f16(q.data_ptr(), k.data_ptr(), v.data_ptr(), self.cos.data_ptr(),
+                                                   self.sin.data_ptr(), self.k_cache[li].data_ptr(),
+                                                   self.v_cache[li].data_ptr(), self.pos.data_ptr(),
+                                                   self.att.data_ptr(), B, H, KV, hd, cfg.max_positions, sp))
+            t = 4 * li                                     # tag bases of this block: t+1 .. t+4
+            ps = [problem(blk.o_proj, self.att, xt, out_tag=t + 1),                                     # x += o_proj(att)
+                  problem(blk.gate_proj, xt, gt, x_tag=t + 1, out_tag=t + 2, norm=blk.post_norm, overwrite=True),
+                  problem(blk.up_proj, xt, ut, x_tag=t + 1, out_tag=t + 3, norm=blk.post_norm, overwrite=True),
+                  problem(blk.down_proj, ut, xt, x_tag=t + 3, gate_tag=t + 2, out_tag=t + 4, gate=gt)]  # x += down(silu(g) * u)
+            if li + 1 < len(self.blocks):
+                nxt = self.blocks[li + 1]
+                ps += [problem(lin, xt, dst, x_tag=t + 4, norm=nxt.input_norm, overwrite=True)
+                       for lin, dst in ((nxt.q_proj, q), (nxt.k_proj, k), (nxt.v_proj, v))]
+            arr = (native.ChainProblem * len(ps))(*ps)
+            check(lib.lutgemm_gemv_rowwise_f16_chain(len(ps), arr, ctypes.byref(ctl), sp))
+        check(lib.lutgemm_chain_untag_rows(x.data_ptr(), xt.data_ptr(), x.numel(), sp))
+        check(lib.lutgemm_chain_advance_epoch(epoch, 4 * len(self.blocks) + 256, sp))
+        check(lib.lutgemm_decode_rmsnorm_f16(x.data_ptr(), self.final_norm.data_ptr(), h.data_ptr(), B, cfg.hidden,
+                                             cfg.rms_eps, None, 0, sp))
+        torch.matmul(h, self.lm_head.t(), out=self.logits)
+
     def _step_hip(self):
+        if self.chain:
+            return self._step_chained()
         cfg, B = self.cfg, self.batch
         hd, H, KV, I = cfg.head_dim, cfg.heads, cfg.kv_heads, cfg.intermediate
         lib = native.cabi()

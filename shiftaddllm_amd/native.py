@@ -15,6 +15,7 @@ import sysconfig
 
 _PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 KERNEL_LIB = os.path.join(_PKG_DIR, "liblutgemm_gfx950.so")
+KERNEL_LIB_TS = os.path.join(_PKG_DIR, "liblutgemm_gfx950_ts.so")
 TORCH_EXT = os.path.join(_PKG_DIR, "lutgemm" + (sysconfig.get_config_var("EXT_SUFFIX") or ".so"))
 
 C_ABI_SYMBOLS = (
@@ -39,6 +40,7 @@ C_ABI_SYMBOLS = (
     "lutgemm_reserve_workspace",
     "lutgemm_describe_plan",
     "lutgemm_set_option",
+    "lutgemm_set_timestamp_buffer",
     "lutgemm_get_option",
     "lutgemm_measure_stream_read",
     "lutgemm_measure_empty_launch",
@@ -51,7 +53,7 @@ C_ABI_SYMBOLS = (
 
 MAX_GROUP = 8
 OPTIONS = {"TARGET_BLOCKS": 0, "FIRST_SHARE": 1, "MFMA_MIN_M": 2, "MFMA_BLOCKS": 3, "PAIR_TABLES": 4, "SINGLE_ITEM": 5,
-           "CHAIN_BLOCKS": 6}
+           "CHAIN_BLOCKS": 6, "CHAIN_GRID": 7}
 CHAIN_MAX_ROWS = 4
 CHAIN_MAX_TAG = 65534
 NOALLOC_MAX_WORDS = 1 << 18
@@ -118,7 +120,70 @@ def _load_extension():
     return module
 
 
+def _bind(lib: ctypes.CDLL) -> ctypes.CDLL:
+    """Set argument and result types of every entry point of include/lutgemm_gfx950.h."""
+    vp, ci, sz = ctypes.c_void_p, ctypes.c_int, ctypes.c_size_t
+    lib.lutgemm_strerror.argtypes = [ci]
+    lib.lutgemm_strerror.restype = ctypes.c_char_p
+    lib.lutgemm_last_hip_error.argtypes = []
+    lib.lutgemm_last_hip_error.restype = ci
+    lib.lutgemm_gemv_rowwise_f16.argtypes = [vp, vp, vp, vp, ci, ci, ci, ci, ci, vp]
+    lib.lutgemm_gemv_rowwise_f16_noalloc.argtypes = [vp, vp, vp, vp, ci, ci, ci, ci, ci, vp]
+    lib.lutgemm_gemv_rowwise_f16_noalloc.restype = ci
+    lib.lutgemm_gemv_rowwise_f16_grouped.argtypes = [ci, ctypes.POINTER(RowwiseProblem), vp]
+    lib.lutgemm_gemv_rowwise_f16_grouped.restype = ci
+    lib.lutgemm_gemv_rowwise_f16_fused.argtypes = [ci, ctypes.POINTER(FusedProblem), vp]
+    lib.lutgemm_gemv_rowwise_f16_fused.restype = ci
+    lib.lutgemm_gemv_rowwise_f16_chain.argtypes = [ci, ctypes.POINTER(ChainProblem), ctypes.POINTER(ChainControl), vp]
+    lib.lutgemm_gemv_rowwise_f16_chain.restype = ci
+    lib.lutgemm_chain_tag_rows.argtypes = [vp, vp, sz, ci, vp, vp]
+    lib.lutgemm_chain_tag_rows.restype = ci
+    lib.lutgemm_chain_untag_rows.argtypes = [vp, vp, sz, vp]
+    lib.lutgemm_chain_untag_rows.restype = ci
+    lib.lutgemm_chain_advance_epoch.argtypes = [vp, ctypes.c_uint, vp]
+    lib.lutgemm_chain_advance_epoch.restype = ci
+    lib.lutgemm_chain_status.argtypes = [vp, vp]
+    lib.lutgemm_chain_status.restype = ci
+    lib.lutgemm_gemv_uniform_f16.argtypes = [vp, vp, vp, vp, vp, ci, ci, ci, ci, ci, vp]
+    lib.lutgemm_gemv_block_f16.argtypes = [vp, vp, vp, vp, ci, ci, ci, ci, ci, vp]
+    lib.lutgemm_gemv_block_shift_u16.argtypes = [vp, vp, vp, vp, ci, ci, ci, ci, ci, ci, vp]
+    lib.lutgemm_gemv_block_apot_i8.argtypes = [vp, vp, vp, vp, ci, ci, ci, ci, ci, ci, vp]
+    for name in ("lutgemm_gemv_rowwise_f16", "lutgemm_gemv_uniform_f16", "lutgemm_gemv_block_f16",
+                 "lutgemm_gemv_block_shift_u16", "lutgemm_gemv_block_apot_i8"):
+        getattr(lib, name).restype = ci
+    lib.lutgemm_algorithmic_bytes.argtypes = [ci, ci, ci, ci, sz, ci]
+    lib.lutgemm_algorithmic_bytes.restype = sz
+    lib.lutgemm_copy_bytes.argtypes = [vp, vp, sz, vp]
+    lib.lutgemm_copy_bytes.restype = ci
+    lib.lutgemm_describe_plan.argtypes = [ci, ci, ci, ci, ci, ci, ctypes.POINTER(Plan)]
+    lib.lutgemm_describe_plan.restype = ci
+    lib.lutgemm_set_option.argtypes = [ci, ci]
+    lib.lutgemm_set_option.restype = ci
+    lib.lutgemm_get_option.argtypes = [ci]
+    lib.lutgemm_get_option.restype = ci
+    lib.lutgemm_workspace_words.argtypes = [ci, ci]
+    lib.lutgemm_workspace_words.restype = sz
+    lib.lutgemm_reserve_workspace.argtypes = [vp, sz]
+    lib.lutgemm_reserve_workspace.restype = ci
+    lib.lutgemm_measure_stream_read.argtypes = [vp, sz, vp, vp]
+    lib.lutgemm_measure_stream_read.restype = ci
+    lib.lutgemm_measure_empty_launch.argtypes = [ci, vp]
+    lib.lutgemm_measure_empty_launch.restype = ci
+    lib.lutgemm_release_workspaces.argtypes = []
+    lib.lutgemm_release_workspaces.restype = ci
+    lib.lutgemm_decode_rmsnorm_f16.argtypes = [vp, vp, vp, ci, ci, ctypes.c_float, vp, sz, vp]
+    lib.lutgemm_decode_rmsnorm_f16.restype = ci
+    lib.lutgemm_decode_attention_f16.argtypes = [vp] * 9 + [ci] * 5 + [vp]
+    lib.lutgemm_decode_attention_f16.restype = ci
+    lib.lutgemm_decode_silu_mul_f16.argtypes = [vp, vp, vp, sz, vp]
+    lib.lutgemm_decode_silu_mul_f16.restype = ci
+    lib.lutgemm_set_timestamp_buffer.argtypes = [vp, sz]
+    lib.lutgemm_set_timestamp_buffer.restype = ci
+    return lib
+
+
 _cabi = None
+_cabi_ts = None
 
 
 def cabi() -> ctypes.CDLL:
@@ -127,64 +192,20 @@ def cabi() -> ctypes.CDLL:
         if not os.path.exists(KERNEL_LIB):
             raise _missing(KERNEL_LIB)
         import torch  # noqa: F401
-        lib = ctypes.CDLL(KERNEL_LIB)
-        vp, ci, sz = ctypes.c_void_p, ctypes.c_int, ctypes.c_size_t
-        lib.lutgemm_strerror.argtypes = [ci]
-        lib.lutgemm_strerror.restype = ctypes.c_char_p
-        lib.lutgemm_last_hip_error.argtypes = []
-        lib.lutgemm_last_hip_error.restype = ci
-        lib.lutgemm_gemv_rowwise_f16.argtypes = [vp, vp, vp, vp, ci, ci, ci, ci, ci, vp]
-        lib.lutgemm_gemv_rowwise_f16_noalloc.argtypes = [vp, vp, vp, vp, ci, ci, ci, ci, ci, vp]
-        lib.lutgemm_gemv_rowwise_f16_noalloc.restype = ci
-        lib.lutgemm_gemv_rowwise_f16_grouped.argtypes = [ci, ctypes.POINTER(RowwiseProblem), vp]
-        lib.lutgemm_gemv_rowwise_f16_grouped.restype = ci
-        lib.lutgemm_gemv_rowwise_f16_fused.argtypes = [ci, ctypes.POINTER(FusedProblem), vp]
-        lib.lutgemm_gemv_rowwise_f16_fused.restype = ci
-        lib.lutgemm_gemv_rowwise_f16_chain.argtypes = [ci, ctypes.POINTER(ChainProblem), ctypes.POINTER(ChainControl), vp]
-        lib.lutgemm_gemv_rowwise_f16_chain.restype = ci
-        lib.lutgemm_chain_tag_rows.argtypes = [vp, vp, sz, ci, vp, vp]
-        lib.lutgemm_chain_tag_rows.restype = ci
-        lib.lutgemm_chain_untag_rows.argtypes = [vp, vp, sz, vp]
-        lib.lutgemm_chain_untag_rows.restype = ci
-        lib.lutgemm_chain_advance_epoch.argtypes = [vp, ctypes.c_uint, vp]
-        lib.lutgemm_chain_advance_epoch.restype = ci
-        lib.lutgemm_chain_status.argtypes = [vp, vp]
-        lib.lutgemm_chain_status.restype = ci
-        lib.lutgemm_gemv_uniform_f16.argtypes = [vp, vp, vp, vp, vp, ci, ci, ci, ci, ci, vp]
-        lib.lutgemm_gemv_block_f16.argtypes = [vp, vp, vp, vp, ci, ci, ci, ci, ci, vp]
-        lib.lutgemm_gemv_block_shift_u16.argtypes = [vp, vp, vp, vp, ci, ci, ci, ci, ci, ci, vp]
-        lib.lutgemm_gemv_block_apot_i8.argtypes = [vp, vp, vp, vp, ci, ci, ci, ci, ci, ci, vp]
-        for name in ("lutgemm_gemv_rowwise_f16", "lutgemm_gemv_uniform_f16", "lutgemm_gemv_block_f16",
-                     "lutgemm_gemv_block_shift_u16", "lutgemm_gemv_block_apot_i8"):
-            getattr(lib, name).restype = ci
-        lib.lutgemm_algorithmic_bytes.argtypes = [ci, ci, ci, ci, sz, ci]
-        lib.lutgemm_algorithmic_bytes.restype = sz
-        lib.lutgemm_copy_bytes.argtypes = [vp, vp, sz, vp]
-        lib.lutgemm_copy_bytes.restype = ci
-        lib.lutgemm_describe_plan.argtypes = [ci, ci, ci, ci, ci, ci, ctypes.POINTER(Plan)]
-        lib.lutgemm_describe_plan.restype = ci
-        lib.lutgemm_set_option.argtypes = [ci, ci]
-        lib.lutgemm_set_option.restype = ci
-        lib.lutgemm_get_option.argtypes = [ci]
-        lib.lutgemm_get_option.restype = ci
-        lib.lutgemm_workspace_words.argtypes = [ci, ci]
-        lib.lutgemm_workspace_words.restype = sz
-        lib.lutgemm_reserve_workspace.argtypes = [vp, sz]
-        lib.lutgemm_reserve_workspace.restype = ci
-        lib.lutgemm_measure_stream_read.argtypes = [vp, sz, vp, vp]
-        lib.lutgemm_measure_stream_read.restype = ci
-        lib.lutgemm_measure_empty_launch.argtypes = [ci, vp]
-        lib.lutgemm_measure_empty_launch.restype = ci
-        lib.lutgemm_release_workspaces.argtypes = []
-        lib.lutgemm_release_workspaces.restype = ci
-        lib.lutgemm_decode_rmsnorm_f16.argtypes = [vp, vp, vp, ci, ci, ctypes.c_float, vp, sz, vp]
-        lib.lutgemm_decode_rmsnorm_f16.restype = ci
-        lib.lutgemm_decode_attention_f16.argtypes = [vp] * 9 + [ci] * 5 + [vp]
-        lib.lutgemm_decode_attention_f16.restype = ci
-        lib.lutgemm_decode_silu_mul_f16.argtypes = [vp, vp, vp, sz, vp]
-        lib.lutgemm_decode_silu_mul_f16.restype = ci
-        _cabi = lib
+        _cabi = _bind(ctypes.CDLL(KERNEL_LIB))
     return _cabi
+
+
+def cabi_timestamps() -> ctypes.CDLL:
+    """The time-stamped build of the library (measurements only: its look-up kernels read the clock
+    at fixed points, see lutgemm_set_timestamp_buffer)."""
+    global _cabi_ts
+    if _cabi_ts is None:
+        if not os.path.exists(KERNEL_LIB_TS):
+            raise _missing(KERNEL_LIB_TS)
+        import torch  # noqa: F401
+        _cabi_ts = _bind(ctypes.CDLL(KERNEL_LIB_TS))
+    return _cabi_ts
 
 
 def __getattr__(name):

@@ -283,3 +283,46 @@ def test_chain_rejects_bad_calls(gpu_device):
     # a well-formed pair still runs
     _ok(_chain([_chain_problem(a, x, t1, M, out_tag=1, overwrite=True), _chain_problem(b, t1, t2, M, x_tag=1, out_tag=2, overwrite=True)], sync))
     assert sync.status() == 0
+
+
+@pytest.mark.parametrize("batch", [1, 2])
+def test_chained_decoder_matches_the_dense_model(gpu_device, batch):
+    """The decoder harness with one chained launch per block (attention kernel + chain) against the
+    same network with every linear a dense fp32 matmul on oracle-dequantised weights, eager and from
+    a captured graph, over several tokens (the epoch advances every step)."""
+    from shiftaddllm_amd import decode, workload
+    cfg = decode.DecoderConfig(vocab_size=512, hidden=256, intermediate=512, layers=3, heads=4, kv_heads=2,
+                               max_positions=32, group_size=128)
+    qc = workload.mixed_bit_config(cfg.layers, seed=3)
+    ids = torch.randint(0, cfg.vocab_size, (batch, 7), generator=torch.Generator().manual_seed(0))
+
+    def run(model, capture):
+        if capture:
+            model.capture()
+        model.reset()
+        outs = []
+        for t in range(ids.shape[1]):
+            outs.append(model.forward_token(ids[:, t].to(gpu_device), t).float().cpu().clone())
+        torch.cuda.synchronize()
+        return torch.stack(outs)
+
+    lut = decode.LutDecoder(cfg, qc, batch=batch, seed=5, device=gpu_device, chain=True)
+    assert lut.chain
+    dense = decode.LutDecoder(cfg, qc, batch=batch, seed=5, device=gpu_device, fuse_launches=False, glue="torch")
+    table = {}
+    for blk in dense.blocks:
+        for lin in (blk.q_proj, blk.k_proj, blk.v_proj, blk.o_proj, blk.gate_proj, blk.up_proj, blk.down_proj):
+            Wq = orc.dequant_rowwise_kernel_layout(lin.binaryWeight.cpu().numpy(), lin.alpha.cpu().numpy())
+            table[id(lin)] = torch.from_numpy(Wq).to(gpu_device)
+    dense._linears = lambda lins, x: [(x.float() @ table[id(l)].t()).half() for l in lins]
+    want = run(dense, capture=False)
+    print(f"chained decoder batch={batch} eager", flush=True)
+    got = run(lut, capture=False)
+    assert lut.chain_status() == 0
+    print(f"chained decoder batch={batch} graph", flush=True)
+    got_graph = run(lut, capture=True)
+    assert lut.chain_status() == 0
+    for name, g in (("eager", got), ("graph", got_graph)):
+        rel, mad = orc.error_metrics(g.numpy(), want.numpy())
+        assert rel <= 2e-3 and mad <= 1e-2, (name, rel, mad)
+    assert torch.allclose(got_graph, got, atol=2e-3, rtol=2e-3)
