@@ -816,15 +816,18 @@ def main():
         decode_res = {}
         qc = workload.mixed_bit_config(decode.LLAMA2_7B.layers, seed=0)
         counts = {b: sum(v["bits"] == b for v in qc.values()) for b in (2, 3, 4)}
-        for B in (1, 8):
-            model = decode.LutDecoder(decode.LLAMA2_7B, qc, batch=B, seed=0, device=dev, fuse_launches=True)
+        for B, chained_step in ((1, False), (8, False), (1, True)):
+            model = decode.LutDecoder(decode.LLAMA2_7B, qc, batch=B, seed=0, device=dev, fuse_launches=True,
+                                      chain=chained_step)
             if not args.no_graph:
                 model.capture()
             prompt = torch.randint(0, decode.LLAMA2_7B.vocab_size, (B, 128),
                                    generator=torch.Generator().manual_seed(0))
             r = decode.benchmark(model, prompt, generate=128, warmup=100)   # 100 warm-up forwards, as model/opt.py:397 does
             lin_bytes = model.linear_bytes_per_token()
-            decode_res[f"batch{B}"] = {
+            if model.chain_status():
+                raise SystemExit("a wait of the chained decode step gave up")
+            decode_res[f"batch{B}" + ("_chained" if chained_step else "")] = {
                 "median_ms_per_token": round(r["median_s_per_token"] * 1e3, 4),
                 "tokens_per_s": round(r["tokens_per_s"], 1),
                 "median_ms_per_prompt_token": round(r["median_s_per_prompt_token"] * 1e3, 4),
@@ -842,7 +845,9 @@ def main():
                                 "launches, SiLU*up folded into the down_proj GEMV (5 launches per block); "
                                 "batch 8: matrix-core kernel, RMSNorm split over the GEMV that completes the "
                                 "residual row and the GEMVs that read it, SiLU*up as a HIP kernel "
-                                "(6 launches per block); embedding gather and fp16 lm_head in torch")
+                                "(6 launches per block); embedding gather and fp16 lm_head in torch; "
+                                "batch1_chained: o_proj, gate/up, down_proj and the next block's q,k,v as ONE chained "
+                                "launch per block (activations handed over through tagged rows), 2 launches per block")
 
     # ---- the reference's real call path: HF OPT -> LutLinear.forward -> lutgemm_compute_block_shiftInt8 ----
     hf_res = None
@@ -856,6 +861,9 @@ def main():
                 traffic = float(line.split(":", 1)[1].strip())
 
     mean_bytes = step_bytes / calls_per_step
+    # Key order: the bulky tables first, the figures a reader of the last kilobyte or two of the line
+    # needs last (per-shape table, fused sequences, decode tokens/s, floors, CPU baseline, roofline).
+    # `roofline` also carries the decode rates, the floors and the fused sequences as flat keys.
     result = {
         "metric": "lut_gemv_us_per_call_llama2_7b_3bit_batch1",
         "value": round(value_us, 4),
@@ -874,30 +882,43 @@ def main():
                                f"({step_bytes / 1e9:.3f} GB/step); " + DATA_NOTE,
                    "launch": launch_mode + ", one launch per GEMV; " + step_kind,
                    "calls_per_step": calls_per_step},
+        "configs": configs,
+        "parity": parity,
+        "hf_opt_call_path": hf_res,
+        "decode_config": decode_res.pop("config") if decode_res else None,
+        "dependency_branches": branched,
+        "pool_build_s": round(t_pool, 2),
+        "device": device_info,
         "device_ms_per_step": round(dev_ms_per_step, 5),
         "achieved_GBps": round(achieved_gbs, 1),
         "frac_hbm_peak": round(achieved_gbs / HBM_PEAK_GBS, 4),
         "decode_tokens_per_s_linears_only": round(1e3 / dev_ms_per_step, 1),
-        "dependency_branches": branched,
-        "roofline": {"bound": "hbm", "achieved": round(achieved_gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(achieved_gbs / HBM_PEAK_GBS, 4), "traffic": traffic,
-                     "kernel": "lut_gemv_kernel<3, 0, 1, false, *> (nb=3, row-wise alpha, 1 row; the 4096x4096 launches, "
-                               "one item per workgroup, take the single-item instance)",
-                     "algorithmic_bytes_per_launch": round(mean_bytes),
-                     "avg_launch_us": round(value_us, 4),
-                     "measured": "224 launches one after the other on one stream (graph replay), HIP events on that stream",
-                     "floors": floors},
-        "cpu_baseline": cpu,
-        "fused_launches": fused,
-        "decode": decode_res,
-        "hf_opt_call_path": hf_res,
-        "configs": configs,
-        "parity": parity,
-        "pool_build_s": round(t_pool, 2),
-        "device": device_info,
     }
     if shape_table is not None:
-        result["shapes"] = shape_table
+        result["shapes"] = {k: {"hot_us": v["hot"]["us_per_call"], "rotating_us": v["rotating"]["us_per_call"],
+                                "rotating_frac_hbm_peak": v["rotating"]["frac_hbm_peak"],
+                                "stream_read_floor_us": v.get("stream_read_floor_us"),
+                                "algorithmic_bytes": v["algorithmic_bytes"]} for k, v in shape_table.items()}
+    result["fused_launches"] = fused
+    result["decode"] = decode_res
+    result["cpu_baseline"] = cpu
+    roof = {"bound": "hbm", "achieved": round(achieved_gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+            "frac": round(achieved_gbs / HBM_PEAK_GBS, 4), "traffic": traffic,
+            "kernel": "lut_gemv_kernel<3, 0, 1, false, *> (nb=3, row-wise alpha, 1 row; the 4096x4096 launches, "
+                      "one item per workgroup, take the single-item instance)",
+            "algorithmic_bytes_per_launch": round(mean_bytes),
+            "avg_launch_us": round(value_us, 4),
+            "measured": "224 launches one after the other on one stream (graph replay), HIP events on that stream"}
+    for k, v in (floors or {}).items():
+        roof["floor_" + k] = v
+    for k, v in fused.items():
+        roof[k + "_frac"] = v["frac_hbm_peak"]
+        roof[k + "_us_per_gemv"] = v["us_per_gemv"]
+    for k, v in (decode_res or {}).items():
+        if isinstance(v, dict):
+            roof[f"decode_{k}_tokens_per_s"] = v["tokens_per_s"]
+            roof[f"decode_{k}_ms_per_token"] = v["median_ms_per_token"]
+    result["roofline"] = roof
     print(json.dumps(result))
 
 

@@ -411,17 +411,21 @@ int lutgemm_gemv_rowwise_f16_fused(int count, const lutgemm_fused_problem *probl
  * (LUTGEMM_EUNSUP).  1 <= M <= LUTGEMM_CHAIN_MAX_ROWS (one row per workgroup,
  * look-up kernel).  Tags lie in 1..LUTGEMM_CHAIN_MAX_TAG.
  *
- * Order.  Workgroups are dispatched problem by problem in the order given, which
- * is what keeps a wait from starving the problem it waits for: a problem must
- * come AFTER every problem of the call whose tag it waits for (LUTGEMM_EINVAL),
- * and problems must be listed stage by stage (those that wait for nothing, then
- * those that wait for them, ...).  A tag that no problem of the call writes is
- * waited for all the same: the row may be written by other work of the process,
- * but nothing guarantees that such work runs while the call waits, so every wait
- * is bounded (control->spin_limit_us, 0 = 100000).  A wait that gives up sets bit
- * 0 of *control->status (device memory, zero before the call); the waiting
- * workgroups of the call then exit without writing, the kernel ends normally,
- * and lutgemm_chain_status() reports LUTGEMM_ETIMEDOUT.
+ * Order.  The launch is persistent: as many workgroups as the device holds of the
+ * kernel at once walk the call's units (one workgroup's range of one problem,
+ * numbered in the order the problems are given) in increasing order, which is
+ * what keeps a wait from starving the problem it waits for (see
+ * lutgemm_describe_chain_plan).  So a problem must come AFTER every problem of
+ * the call whose tag it waits for (LUTGEMM_EINVAL), and problems must be listed
+ * stage by stage (those that wait for nothing, then those that wait for them,
+ * ...).  A tag that no problem of the call writes is waited for all the same:
+ * the row may be written by other work of the process, but nothing guarantees
+ * that such work runs while the call waits, and kernels of other streams that
+ * run at the same time may keep part of the launch from being resident, so every
+ * wait is bounded (control->spin_limit_us, 0 = 100000).  A wait that gives up
+ * sets bit 0 of *control->status (device memory, zero before the call); the
+ * waiting workgroups of the call then exit without writing, the kernel ends
+ * normally, and lutgemm_chain_status() reports LUTGEMM_ETIMEDOUT.
  *
  * Epoch.  A captured launch is replayed with the same tags, and last replay's
  * rows would satisfy this replay's waits: the effective tag of base t is
@@ -453,6 +457,28 @@ typedef struct lutgemm_chain_control {
 
 int lutgemm_gemv_rowwise_f16_chain(int count, const lutgemm_chain_problem *problems,
                                    const lutgemm_chain_control *control, void *stream);
+
+/*
+ * How a chained call would be launched (pure host arithmetic when `workgroups` > 0; with 0 the
+ * device is asked how many workgroups of the kernel it holds at once, which is what the compute
+ * call uses).  The launch is persistent: `workgroups` workgroups, all resident at the same time,
+ * take the call's `units` (one workgroup's range of one problem, numbered problem by problem in
+ * the order given) in steps of `workgroups`: workgroup w takes units w, w + workgroups, ...
+ * A unit waits only for units with smaller numbers, and every workgroup takes its units in
+ * increasing order, so the unfinished unit with the smallest number can always run: no wait can
+ * starve the unit it waits for.  That argument needs every workgroup of the launch resident,
+ * which other kernels running at the same time can prevent: hence the bounded waits.
+ * Per problem: its stage (0 = waits for nothing in the call), its first unit, its units, and the
+ * (tile, set) items of a unit (the last unit of a problem may hold fewer).  Returns what the
+ * compute call would return for the same problems without launching anything.
+ */
+typedef struct lutgemm_chain_plan {
+    int workgroups, units, needs_workspace;
+    int stage[LUTGEMM_MAX_GROUP], first_unit[LUTGEMM_MAX_GROUP], unit_count[LUTGEMM_MAX_GROUP],
+        items_per_unit[LUTGEMM_MAX_GROUP];
+} lutgemm_chain_plan;
+int lutgemm_describe_chain_plan(int count, const lutgemm_chain_problem *problems, int workgroups,
+                                lutgemm_chain_plan *plan);
 
 /* dst_tagged[i] = src_f16[i] | effective tag << 16 (count values), and back. */
 int lutgemm_chain_tag_rows(void *dst_tagged, const void *src_f16, size_t count, int tag, const uint32_t *epoch,

@@ -659,15 +659,15 @@ int chain_grid(int *out)
     return LUTGEMM_OK;
 }
 
-int run_chain(int count, const lutgemm_chain_problem *problems, const lutgemm_chain_control *ctl, const Accum &acc)
+// Validate the problems of a chained launch and cut them into units (no device work when
+// grid_in > 0).  On return c.g holds the planned problems, c.unit_start the units, depth[] the
+// stage of every problem, *grid the workgroups of the launch.
+int plan_chain(int count, const lutgemm_chain_problem *problems, int grid_in, Chain &c, int *depth, int *grid_out,
+               bool *any_split_out, size_t *words_out)
 {
-    if (!ctl || !ctl->status) return LUTGEMM_EINVAL;
-    if (!aligned(ctl->status, 4) || !aligned(ctl->epoch, 4)) return LUTGEMM_EALIGN;
-    Chain c{};
     Group &g = c.g;
     g.count = count;
     size_t words = 0;
-    int depth[kMaxGroup];
     unsigned direct[kMaxGroup], after[kMaxGroup], before_inputs[kMaxGroup];
     for (int i = 0; i < count; ++i) {
         const lutgemm_chain_problem &cq = problems[i];
@@ -758,8 +758,8 @@ int run_chain(int count, const lutgemm_chain_problem *problems, const lutgemm_ch
     }
     // Plan stage by stage: the problems of a stage share one round of the grid (every workgroup
     // takes one unit of the stage) unless LUTGEMM_OPTION_CHAIN_BLOCKS says otherwise.
-    int grid = 0;
-    {
+    int grid = grid_in;
+    if (grid <= 0) {
         int rc = chain_grid(&grid);
         if (rc != LUTGEMM_OK) return rc;
     }
@@ -775,15 +775,48 @@ int run_chain(int count, const lutgemm_chain_problem *problems, const lutgemm_ch
             bytes += (long)g.p[last].N * (g.p[last].K / 8) * g.p[last].nb * g.p[last].M;
             ++last;
         }
-        int rc = share_workgroups(ps, last - first, (long)stage_blocks, &begin, &any_split);
-        if (rc != LUTGEMM_OK) return rc;
+        // a range's activations are fetched as one window of sixteen items: a stage whose units
+        // would hold more takes further rounds of the grid
+        constexpr int kWindowItems = kThreads / kTables;
+        for (long rounds = 1;; ++rounds) {
+            bool split = false;
+            int rc = share_workgroups(ps, last - first, rounds * (long)stage_blocks, &begin, &split);
+            if (rc != LUTGEMM_OK) return rc;
+            bool fits = true;
+            for (int i = first; i < last; ++i) fits = fits && g.p[i].items_per_wg <= kWindowItems;
+            if (fits) {
+                any_split = any_split || split;
+                break;
+            }
+            if (rounds >= 4096) return LUTGEMM_EUNSUP;
+        }
         first = last;
     }
-    for (int i = 0; i < count; ++i)   // a range's activations are fetched as one window
-        if (g.p[i].items_per_wg > kThreads / kTables) return LUTGEMM_EUNSUP;
+    c.unit_start[0] = 0;
+    for (int i = 0; i < count; ++i) c.unit_start[i + 1] = c.unit_start[i] + g.p[i].n_blocks;
+    for (int i = count; i < kMaxGroup; ++i) c.unit_start[i + 1] = c.unit_start[count];
+    const int total_units = c.unit_start[count];
+    *grid_out = total_units < grid ? total_units : grid;
+    *any_split_out = any_split;
+    *words_out = words;
+    (void)begin;
+    return LUTGEMM_OK;
+}
+
+int run_chain(int count, const lutgemm_chain_problem *problems, const lutgemm_chain_control *ctl, const Accum &acc)
+{
+    if (!ctl || !ctl->status) return LUTGEMM_EINVAL;
+    if (!aligned(ctl->status, 4) || !aligned(ctl->epoch, 4)) return LUTGEMM_EALIGN;
+    Chain c{};
+    Group &g = c.g;
+    int depth[kMaxGroup], grid = 0;
+    bool any_split = false;
+    size_t words = 0;
+    int rc = plan_chain(count, problems, 0, c, depth, &grid, &any_split, &words);
+    if (rc != LUTGEMM_OK) return rc;
     if (any_split) {
         unsigned long long *base = nullptr;
-        int rc = accum_words(acc, words, &base);
+        rc = accum_words(acc, words, &base);
         if (rc != LUTGEMM_OK) return rc;
         size_t off = 0;
         for (int i = 0; i < count; ++i) {
@@ -795,11 +828,7 @@ int run_chain(int count, const lutgemm_chain_problem *problems, const lutgemm_ch
     c.ctl.status = ctl->status;
     const unsigned us = ctl->spin_limit_us ? ctl->spin_limit_us : 100000u;
     c.ctl.spin_ticks = (long long)us * 100;   // the wall clock ticks at 100 MHz
-    c.unit_start[0] = 0;
-    for (int i = 0; i < count; ++i) c.unit_start[i + 1] = c.unit_start[i] + g.p[i].n_blocks;
-    for (int i = count; i < kMaxGroup; ++i) c.unit_start[i + 1] = c.unit_start[count];
-    const int total_units = c.unit_start[count];
-    const hipError_t e = launch_gemv_chain(c, total_units < grid ? total_units : grid, acc.stream);
+    const hipError_t e = launch_gemv_chain(c, grid, acc.stream);
     return e == hipSuccess ? LUTGEMM_OK : hip_fail(e);
 }
 
@@ -975,6 +1004,29 @@ int lutgemm_gemv_rowwise_f16_chain(int count, const lutgemm_chain_problem *probl
 {
     if (!problems || count < 1 || count > kMaxGroup) return LUTGEMM_EINVAL;
     return run_chain(count, problems, control, Accum{(hipStream_t)stream_v});
+}
+
+int lutgemm_describe_chain_plan(int count, const lutgemm_chain_problem *problems, int workgroups,
+                                lutgemm_chain_plan *plan)
+{
+    if (!problems || !plan || count < 1 || count > kMaxGroup || workgroups < 0) return LUTGEMM_EINVAL;
+    Chain c{};
+    int depth[kMaxGroup], grid = 0;
+    bool any_split = false;
+    size_t words = 0;
+    const int rc = plan_chain(count, problems, workgroups, c, depth, &grid, &any_split, &words);
+    if (rc != LUTGEMM_OK) return rc;
+    *plan = lutgemm_chain_plan{};
+    plan->workgroups = grid;
+    plan->units = c.unit_start[count];
+    plan->needs_workspace = any_split;
+    for (int i = 0; i < count; ++i) {
+        plan->stage[i] = depth[i];
+        plan->first_unit[i] = c.unit_start[i];
+        plan->unit_count[i] = c.g.p[i].n_blocks;
+        plan->items_per_unit[i] = c.g.p[i].items_per_wg;
+    }
+    return LUTGEMM_OK;
 }
 
 int lutgemm_chain_tag_rows(void *dst_tagged, const void *src_f16, size_t count, int tag, const uint32_t *epoch,

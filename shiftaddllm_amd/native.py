@@ -26,6 +26,7 @@ C_ABI_SYMBOLS = (
     "lutgemm_gemv_rowwise_f16_grouped",
     "lutgemm_gemv_rowwise_f16_fused",
     "lutgemm_gemv_rowwise_f16_chain",
+    "lutgemm_describe_chain_plan",
     "lutgemm_chain_tag_rows",
     "lutgemm_chain_untag_rows",
     "lutgemm_chain_advance_epoch",
@@ -95,6 +96,13 @@ class ChainControl(ctypes.Structure):
     _fields_ = [("epoch", ctypes.c_void_p), ("status", ctypes.c_void_p), ("spin_limit_us", ctypes.c_uint)]
 
 
+class ChainPlan(ctypes.Structure):
+    """struct lutgemm_chain_plan of include/lutgemm_gfx950.h."""
+    _fields_ = [("workgroups", ctypes.c_int), ("units", ctypes.c_int), ("needs_workspace", ctypes.c_int),
+                ("stage", ctypes.c_int * MAX_GROUP), ("first_unit", ctypes.c_int * MAX_GROUP),
+                ("unit_count", ctypes.c_int * MAX_GROUP), ("items_per_unit", ctypes.c_int * MAX_GROUP)]
+
+
 class NativeLibraryMissing(ImportError):
     pass
 
@@ -136,6 +144,8 @@ def _bind(lib: ctypes.CDLL) -> ctypes.CDLL:
     lib.lutgemm_gemv_rowwise_f16_fused.restype = ci
     lib.lutgemm_gemv_rowwise_f16_chain.argtypes = [ci, ctypes.POINTER(ChainProblem), ctypes.POINTER(ChainControl), vp]
     lib.lutgemm_gemv_rowwise_f16_chain.restype = ci
+    lib.lutgemm_describe_chain_plan.argtypes = [ci, ctypes.POINTER(ChainProblem), ci, ctypes.POINTER(ChainPlan)]
+    lib.lutgemm_describe_chain_plan.restype = ci
     lib.lutgemm_chain_tag_rows.argtypes = [vp, vp, sz, ci, vp, vp]
     lib.lutgemm_chain_tag_rows.restype = ci
     lib.lutgemm_chain_untag_rows.argtypes = [vp, vp, sz, vp]

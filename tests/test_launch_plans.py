@@ -183,3 +183,99 @@ def test_tuning_options_change_plans_and_keep_their_invariants(lib):
         for k, v in opt.items():
             lib.lutgemm_set_option(v, -1)
     assert {k: lib.lutgemm_get_option(v) for k, v in opt.items()} == start
+
+
+# ---- chained launches: the forward-progress argument as host arithmetic ---------------------------
+
+def _chain_problem(base, N, K, nb, x, out, M=1, x_tag=0, gate_tag=0, out_tag=0, gate=None, norm=None, overwrite=0):
+    from shiftaddllm_amd import native
+    f = native.FusedProblem(base, base + 0x100000, x, out, N, K, nb, K // 128, M, overwrite, norm, gate, 1e-5)
+    return native.ChainProblem(f, x_tag, gate_tag, out_tag)
+
+
+def _decoder_block_chain(hidden, inter, nbs, M=1):
+    """o_proj -> gate, up -> down_proj -> q, k, v of the next block (dummy, never dereferenced addresses)."""
+    A = 0x10000000
+    att, xt, gt, ut, q, k, v, w = (A + i * 0x1000000 for i in range(1, 9))
+    return [_chain_problem(A, hidden, hidden, nbs[0], att, xt, M, out_tag=1),
+            _chain_problem(A, inter, hidden, nbs[1], xt, gt, M, x_tag=1, out_tag=2, norm=w, overwrite=1),
+            _chain_problem(A, inter, hidden, nbs[2], xt, ut, M, x_tag=1, out_tag=3, norm=w, overwrite=1),
+            _chain_problem(A, hidden, inter, nbs[3], ut, xt, M, x_tag=3, gate_tag=2, out_tag=4, gate=gt),
+            _chain_problem(A, hidden, hidden, nbs[4], xt, q, M, x_tag=4, norm=w, overwrite=1),
+            _chain_problem(A, hidden // 4, hidden, nbs[5], xt, k, M, x_tag=4, norm=w, overwrite=1),
+            _chain_problem(A, hidden // 4, hidden, nbs[6], xt, v, M, x_tag=4, norm=w, overwrite=1)]
+
+
+def _describe_chain(lib, problems, workgroups):
+    from shiftaddllm_amd import native
+    arr = (native.ChainProblem * len(problems))(*problems)
+    plan = native.ChainPlan()
+    rc = lib.lutgemm_describe_chain_plan(len(problems), arr, workgroups, ctypes.byref(plan))
+    return rc, plan
+
+
+@pytest.mark.parametrize("workgroups", [64, 256, 512])
+@pytest.mark.parametrize("hidden,inter,nbs,M", [(4096, 11008, (3,) * 7, 1), (4096, 11008, (2, 4, 3, 3, 4, 2, 3), 2),
+                                                (1024, 2688, (3, 2, 4, 3, 2, 3, 4), 1), (8192, 28672, (4,) * 7, 1)])
+def test_chain_plans_cannot_starve_a_producer(lib, workgroups, hidden, inter, nbs, M):
+    """Workgroup w of a chained launch takes units w, w + G, w + 2G, ... in that order, and a unit waits
+    only for units of problems that come earlier in the call.  Checked on the plans: units are numbered
+    problem by problem without gaps, every problem a unit waits for has all its units below the
+    waiter's first unit, stages never decrease, and a unit's items fit one activation window.  Then the
+    schedule is simulated: at every moment the unfinished unit with the smallest number is at the
+    head of its workgroup's queue and everything it waits for has finished."""
+    problems = _decoder_block_chain(hidden, inter, nbs, M)
+    rc, plan = _describe_chain(lib, problems, workgroups)
+    assert rc == 0
+    n = len(problems)
+    G = plan.workgroups
+    assert 1 <= G <= workgroups
+    first = [plan.first_unit[i] for i in range(n)]
+    count = [plan.unit_count[i] for i in range(n)]
+    stage = [plan.stage[i] for i in range(n)]
+    assert first[0] == 0 and all(first[i + 1] == first[i] + count[i] for i in range(n - 1))
+    assert plan.units == first[-1] + count[-1] and all(c >= 1 for c in count)
+    assert stage == sorted(stage) and stage == [0, 1, 1, 2, 3, 3, 3]
+    assert all(1 <= plan.items_per_unit[i] <= 16 for i in range(n))
+    waits_for = {1: [0], 2: [0], 3: [1, 2], 4: [3], 5: [3], 6: [3]}          # by construction of the block
+    for i, ps in waits_for.items():
+        for p in ps:
+            assert first[p] + count[p] <= first[i], "a producer's units all come before its consumers'"
+    # simulate: units finish in some order compatible with "a unit runs when it is at the head of its
+    # workgroup's queue and its producers are done"; the smallest unfinished unit must always be runnable
+    owner_of = lambda u: u % G
+    problem_of = lambda u: max(i for i in range(n) if first[i] <= u)
+    done = [False] * plan.units
+    head = list(range(min(G, plan.units)))                                    # next unit of every workgroup
+    for step in range(plan.units):
+        u = step                                                               # the smallest unfinished unit
+        assert head[owner_of(u)] == u, "its workgroup has finished everything before it"
+        for p in waits_for.get(problem_of(u), []):
+            assert all(done[first[p]:first[p] + count[p]])
+        done[u] = True
+        head[owner_of(u)] = u + G
+
+
+def test_chain_plan_validation_on_the_host(lib):
+    A = 0x10000000
+    x, t1, t2, o = A + 0x1000000, A + 0x2000000, A + 0x3000000, A + 0x4000000
+    ok = [_chain_problem(A, 512, 512, 3, x, t1, out_tag=1, overwrite=1),
+          _chain_problem(A, 512, 512, 3, t1, t2, x_tag=1, out_tag=2, overwrite=1)]
+    rc, plan = _describe_chain(lib, ok, 512)
+    assert rc == 0 and plan.stage[0] == 0 and plan.stage[1] == 1 and plan.needs_workspace in (0, 1)
+    # the consumer listed before its producer
+    assert _describe_chain(lib, ok[::-1], 512)[0] == -1
+    # two writers of one plain row; of one tagged row without an ordering wait
+    assert _describe_chain(lib, [_chain_problem(A, 512, 512, 3, x, o), _chain_problem(A, 512, 512, 3, x, o)], 512)[0] == -1
+    assert _describe_chain(lib, [_chain_problem(A, 512, 512, 3, x, t1, out_tag=1),
+                                 _chain_problem(A, 512, 512, 3, x, t1, out_tag=2)], 512)[0] == -1
+    # accumulating into a row right behind its writer
+    assert _describe_chain(lib, [_chain_problem(A, 512, 512, 3, x, t1, out_tag=1),
+                                 _chain_problem(A, 512, 512, 3, t1, t1, x_tag=1, out_tag=2)], 512)[0] == -1
+    # tags out of range, rows beyond the limit, a tagged norm row wider than 8192
+    assert _describe_chain(lib, [_chain_problem(A, 512, 512, 3, x, t1, out_tag=70000)], 512)[0] == -1
+    assert _describe_chain(lib, [_chain_problem(A, 512, 512, 3, x, o, M=8)], 512)[0] == -3
+    assert _describe_chain(lib, [_chain_problem(A, 512, 16384, 3, t1, o, x_tag=5, norm=x)], 512)[0] == -3
+    # units of more than sixteen items would not fit one activation window: the stage takes more rounds
+    rc, plan = _describe_chain(lib, [_chain_problem(A, 8192, 8192, 3, x, o)], 8)
+    assert rc == 0 and plan.workgroups == 8 and plan.items_per_unit[0] <= 16 and plan.unit_count[0] >= 64
