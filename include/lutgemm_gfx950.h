@@ -235,7 +235,7 @@ typedef struct lutgemm_plan {
     int workgroups;      /* of the launch */
     int rows_per_pass;   /* activation rows a workgroup handles together */
     int row_chunks;      /* ceil(M / rows_per_pass) */
-    int tiles;           /* output tiles: 256 columns (look-up), 64 (matrix cores) */
+    int tiles;           /* output tiles of tile_columns columns */
     int k_units;         /* sets of 256 inputs (look-up), steps of 128 (matrix cores) */
     /* look-up kernel: the tiles x k_units items of a row chunk, tile-major, are cut into
      * `ranges` contiguous ranges: the first `long_ranges` of `items_per_long_range`
@@ -245,6 +245,7 @@ typedef struct lutgemm_plan {
      * `units_per_slice` steps (the last one may be shorter) */
     int k_slices, units_per_slice;
     int needs_workspace; /* 1: the launch uses lutgemm_workspace_words(N, M) accumulator words */
+    int tile_columns;    /* output columns per tile: 256 (look-up), 512 (look-up, twin items), 64 (matrix cores) */
 } lutgemm_plan;
 
 int lutgemm_describe_plan(int format, int N, int K, int nb, int groups, int M, lutgemm_plan *plan);
@@ -267,6 +268,9 @@ int lutgemm_describe_plan(int format, int N, int K, int nb, int groups, int M, l
  *                   kernel, 0 = one fp32 table set per row
  *   SINGLE_ITEM   : 1 = launches whose ranges all hold one item take the kernel
  *                   instance that requests nothing beyond it, 0 = the general one
+ *   TWIN_ITEMS    : one-row look-up launches whose workgroups would all hold at least this
+ *                   many items take twin items instead (one table build per 512 outputs
+ *                   instead of per 256; default 4, 0 = never)
  *   CHAIN_GRID    : workgroups of a chained launch (0 = as many as the device holds
  *                   at once, which is also the upper limit)
  *   CHAIN_BLOCKS  : ranges the problems of one stage of a chained launch are cut into
@@ -280,7 +284,8 @@ int lutgemm_describe_plan(int format, int N, int K, int nb, int groups, int M, l
 #define LUTGEMM_OPTION_SINGLE_ITEM 5
 #define LUTGEMM_OPTION_CHAIN_BLOCKS 6
 #define LUTGEMM_OPTION_CHAIN_GRID 7
-#define LUTGEMM_OPTION_COUNT 8
+#define LUTGEMM_OPTION_TWIN_ITEMS 8
+#define LUTGEMM_OPTION_COUNT 9
 int lutgemm_set_option(int which, int value);
 int lutgemm_get_option(int which);
 

@@ -673,8 +673,11 @@ __device__ __forceinline__ float reduce_scatter_kw(const float (&acc)[4], int kw
 // DEP: a problem of a chained launch (`cw` non-null): x, gate and out may be tagged rows.  The
 //      operands that depend on nothing (sign words and alphas of the first two items) are
 //      requested at once; the activations are waited for, tag by tag, behind them.
+// TWIN: the items are "twin" items: the same set of 256 inputs against TWO neighbouring output
+//       tiles (512 outputs), so that one table build and one barrier serve two look-up passes.
+//       The problem's n_tiles counts tile pairs then, and the planner's items are twin items.
 template <int NB, int MODE, int MROWS, int XF = kXNone, bool EXTRA = false, int ALONE = MROWS == 1 && !is_block(MODE),
-          bool PAIR = false, bool DEP = false>
+          bool PAIR = false, bool DEP = false, bool TWIN = false>
 __device__ __forceinline__ bool gemv_range(const Problem &p, int range, int mchunk, float *lut, const ChainWait *cw = nullptr)
 {
     // Returns false when a chained problem gave up waiting for its inputs (nothing was written).
@@ -688,6 +691,8 @@ __device__ __forceinline__ bool gemv_range(const Problem &p, int range, int mchu
     static_assert(!(EXTRA || XF == kXNorm) || !is_staged(MODE), "the per-wave sums live in the alpha staging area");
     static_assert(!DEP || (MROWS == 1 && MODE == kRowF16 && !EXTRA && !PAIR), "chained launches: one row per workgroup, row-wise alphas");
     static_assert(DEP == (XF == kXDynamic), "chained problems choose their transform at run time, the others at compile time");
+    static_assert(!TWIN || (MROWS == 1 && ALONE == 1 && !EXTRA && !PAIR && !DEP), "twin items: one row, first item alone, no extras");
+    constexpr int kMembers = TWIN ? 2 : 1;   // output tiles per item
     // the transform: a compile-time constant except for chained problems (one kernel holds them
     // all, and an instance per bit width and transform is more than the compiler digests: from
     // eight instances of this function on, it emits an empty kernel)
@@ -724,6 +729,7 @@ __device__ __forceinline__ bool gemv_range(const Problem &p, int range, int mchu
     for (int r = 0; r < MROWS; ++r)
 #pragma unroll
         for (int i = 0; i < 4; ++i) acc[r][i] = 0.0f;
+    [[maybe_unused]] float acc_twin[4] = {0.0f, 0.0f, 0.0f, 0.0f};   // the item's second tile
 
     // table-build role of this thread
     const int tb = tid & 31;  // table (bank)
@@ -861,7 +867,17 @@ __device__ __forceinline__ bool gemv_range(const Problem &p, int range, int mchu
     // the caller's output, needed only by whoever completes a sum: fetched early,
     // off the critical path (again whenever the range moves on to another tile)
     unsigned short out_prev[MROWS];
+    [[maybe_unused]] unsigned short out_prev_twin = 0;
     auto fetch_out = [&](int t) {
+        if constexpr (TWIN) {
+            // t counts tile pairs
+            const int na = min(2 * t * kTileCols + own_col_of(kw), p.N - 1);
+            const int nb2 = min((2 * t + 1) * kTileCols + own_col_of(kw), p.N - 1);
+            const unsigned short *row = (const unsigned short *)(p.out + (size_t)min(m0, p.M - 1) * p.N);
+            out_prev[0] = row[na];
+            out_prev_twin = row[nb2];
+            return;
+        }
         const int n = min(t * kTileCols + own_col_of(kw), p.N - 1);
         if constexpr (DEP) {
             // a tagged row that an earlier problem of the launch may have completed: its values
@@ -959,8 +975,46 @@ __device__ __forceinline__ bool gemv_range(const Problem &p, int range, int mchu
         const int count = range_of(t * p.nsets + p.nsets - 1) - range_of(t * p.nsets) + 1;
         int kw2 = kw;
         asm volatile("" : "+v"(kw2));  // (opaque: see own_col_of)
-        const int n = t * kTileCols + own_col_of(kw2);
         const bool owner = (kw2 & 1) == 0;
+        if constexpr (TWIN) {
+            // both tiles of the pair (one row, no extras): both atomics are issued before either
+            // result is looked at, so that their round trips overlap
+            int n2[2];
+            float v2[2];
+            Contribution c2[2];
+            unsigned long long old2[2] = {0ull, 0ull};
+            bool mine[2];
+#pragma unroll
+            for (int member = 0; member < 2; ++member) {
+                n2[member] = (2 * t + member) * kTileCols + own_col_of(kw2);
+                v2[member] = reduce_scatter_kw(member ? acc_twin : acc[0], kw2);
+#pragma unroll
+                for (int i = 0; i < 4; ++i) (member ? acc_twin : acc[0])[i] = 0.0f;
+                mine[member] = owner && n2[member] < p.N;
+                c2[member] = fixed_contribution(v2[member]);
+                if (mine[member] && count > 1) {
+                    unsigned long long *word = p.accum + (size_t)m0 * p.N + n2[member];
+                    if (c2[member].flags)
+                        __hip_atomic_fetch_or(word, c2[member].flags, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    old2[member] = __hip_atomic_fetch_add(word, c2[member].add, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                }
+            }
+#pragma unroll
+            for (int member = 0; member < 2; ++member) {
+                if (!mine[member]) continue;
+                __half *dst = p.out + (size_t)m0 * p.N + n2[member];
+                const float prev = p.overwrite ? 0.0f : half_bits_to_float(member ? out_prev_twin : out_prev[0]);
+                if (count == 1) {
+                    *dst = __float2half_rn(prev + v2[member]);
+                    continue;
+                }
+                if ((int)(old2[member] >> 56) != count - 1) continue;
+                *dst = __float2half_rn(prev + fixed_total((old2[member] | c2[member].flags) + c2[member].add, count));
+                __hip_atomic_store(p.accum + (size_t)m0 * p.N + n2[member], 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+            return;
+        }
+        const int n = t * kTileCols + own_col_of(kw2);
         bool scaled = xf == kXNorm;
         if constexpr (EXTRA) scaled = scaled || p.sumsq_in != nullptr;
         // the next norm's weight for this lane's column: requested here, used once the
@@ -1035,6 +1089,25 @@ __device__ __forceinline__ bool gemv_range(const Problem &p, int range, int mchu
     int buf = 0;
     int rel = 0;  // items of the range done so far
     // `after_first_barrier` runs behind the barrier of the item's first row (see the first item below).
+    // Twin items: the item's second tile is looked up against the tables that stand already.
+    [[maybe_unused]] auto twin_second = [&](const ItemOperands<NB, MODE> &ops, bool last) {
+        int nt = tile, ns = set;
+        advance(nt, ns);
+        asm volatile("" : "+v"(lane_off));
+        lookup_item<NB, MODE>(ops, lut, acc_twin, lane_off, sel, stage + abuf * (2 * 4 * kTables) + kw * 4, q);
+        buf ^= 1;
+        lane_off ^= kFlip;
+        if (rel == 0) stamp(p, kStampFirstItem);
+        ++rel;
+        if (last) stamp(p, kStampItems);
+        if (last || nt != tile) {
+            flush_tile(tile);
+            if (!last) fetch_out(nt);
+        }
+        if (last) stamp(p, kStampHandedOver);
+        tile = nt;
+        set = ns;
+    };
     auto item_step = [&](const ItemOperands<NB, MODE> &ops, bool last, auto &&after_first_barrier) {
         int nt = tile, ns = set;
         advance(nt, ns);
@@ -1090,6 +1163,7 @@ __device__ __forceinline__ bool gemv_range(const Problem &p, int range, int mchu
             // kept in registers across all rows instead of being recomputed (1 op each)
             asm volatile("" : "+v"(lane_off));
             lookup_item<NB, MODE>(ops, lut, acc[r], lane_off, sel, stage + abuf * (2 * 4 * kTables) + kw * 4, q);
+            if constexpr (TWIN) return;   // (the buffers turn, and the range moves on, behind the second tile)
             buf ^= 1;
             lane_off ^= kFlip;
         }
@@ -1146,6 +1220,29 @@ __device__ __forceinline__ bool gemv_range(const Problem &p, int range, int mchu
         first_window();
         load_item<NB, MODE, 2>(opA, p, ld_tile, ld_set, true, kw, q, lane_col, tid);
         item_step(opA, true, [&]() { fetch_out(tile); });
+    } else if constexpr (TWIN) {
+        // Twin items: buffer A holds the item's first tile, buffer B its second.  The first tile's
+        // step builds the tables (first item alone, as below), the second tile's step only looks up.
+        load_item<NB, MODE, 1>(opA, p, 2 * ld_tile, ld_set, true, kw, q, lane_col, tid);
+        __builtin_amdgcn_sched_barrier(0);
+        stamp(p, kStampRequested);
+        late_setup();
+        first_window();
+        load_item<NB, MODE, 2>(opA, p, 2 * ld_tile, ld_set, true, kw, q, lane_col, tid);
+        item_step(opA, false, [&]() {
+            fetch_out(tile);
+            load_item<NB, MODE>(opB, p, 2 * ld_tile + 1, ld_set, true, kw, q, lane_col, tid);
+            advance(ld_tile, ld_set);
+        });
+#pragma clang loop unroll(disable)
+        for (int j = 1; j < n_items; ++j) {
+            load_item<NB, MODE>(opA, p, 2 * ld_tile, ld_set, true, kw, q, lane_col, tid);
+            twin_second(opB, false);
+            load_item<NB, MODE>(opB, p, 2 * ld_tile + 1, ld_set, true, kw, q, lane_col, tid);
+            advance(ld_tile, ld_set);
+            item_step(opA, false, no_hook);
+        }
+        twin_second(opB, true);
     } else if constexpr (ALONE == 1) {
         load_item<NB, MODE, 1>(opA, p, ld_tile, ld_set, true, kw, q, lane_col, tid);
         __builtin_amdgcn_sched_barrier(0);
@@ -1226,13 +1323,15 @@ __device__ __forceinline__ void decode_block(const Problem &p, int local, int &r
 
 // (at most 128 registers, so that two workgroups share a CU)
 // SINGLE: every range of the launch holds exactly one item (see ALONE == 2 in gemv_range).
-template <int NB, int MODE, int MROWS, bool PAIR = false, bool SINGLE = false>
+// TWIN: the launch's items are twin items (two output tiles per table build, see gemv_range).
+template <int NB, int MODE, int MROWS, bool PAIR = false, bool SINGLE = false, bool TWIN = false>
 __global__ void __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4, 4)))
 lut_gemv_kernel(const Problem p)
 {
     __shared__ __attribute__((aligned(16))) float lut[kLutDwords + kStageDwords + kWindowDwords];
     // grid = (ranges, row chunks)
-    gemv_range<NB, MODE, MROWS, kXNone, false, SINGLE ? 2 : (MROWS == 1 && !is_block(MODE)), PAIR>(p, (int)blockIdx.x, (int)blockIdx.y, lut);
+    gemv_range<NB, MODE, MROWS, kXNone, false, SINGLE ? 2 : (MROWS == 1 && !is_block(MODE)), PAIR, false, TWIN>(
+        p, (int)blockIdx.x, (int)blockIdx.y, lut);
 }
 
 // Several row-wise problems in one launch.  Bit widths may differ between the

@@ -26,6 +26,8 @@ hipError_t launch_nb(const Problem &p, int mrows, hipStream_t stream)
         hipLaunchKernelGGL((lut_gemv_kernel<NB, MODE, 4>), grid, block, 0, stream, p);
     else if (mrows == 2)
         hipLaunchKernelGGL((lut_gemv_kernel<NB, MODE, 2>), grid, block, 0, stream, p);
+    else if (p.twin)
+        hipLaunchKernelGGL((lut_gemv_kernel<NB, MODE, 1, false, false, true>), grid, block, 0, stream, p);
     else if (p.items_per_wg == 1 && p.short_items == 1 && single_item)
         hipLaunchKernelGGL((lut_gemv_kernel<NB, MODE, 1, false, true>), grid, block, 0, stream, p);
     else

@@ -24,7 +24,8 @@ constexpr int kTileCols = kWaves * kWaveCols;  // outputs a workgroup covers (25
 constexpr int kEntryStride = 64;           // dwords between consecutive entries of a table
 constexpr int kLutDwords = 256 * kEntryStride;  // 64 KiB: two interleaved table buffers
 constexpr int kStageDwords = 2 * 2 * 4 * kTables;  // staged block alphas: [buffer][row group][bit][chunk]
-constexpr int kMaxContrib = 32;            // contributions per accumulator word (see below)
+constexpr int kMaxContrib = 40;            // contributions per accumulator word (see below)
+constexpr int kMaxSlices = 32;             // matrix-core kernel: K-slices per tile
 constexpr int kMaxGroup = LUTGEMM_MAX_GROUP;  // problems per grouped launch
 
 // Fixed-point accumulator word of one output (K split over workgroups):
@@ -32,7 +33,7 @@ constexpr int kMaxGroup = LUTGEMM_MAX_GROUP;  // problems per grouped launch
 //   [55]    a contribution was -inf, below -2^16, or NaN
 //   [54]    a contribution was +inf, above +2^16, or NaN
 //   [53:0]  sum of (v + kBias), v = partial * 2^31 rounded, |partial| <= 2^16
-// kMaxContrib contributions of at most 2^48 + 2^47 stay below 2^54.  Integer
+// kMaxContrib contributions of at most 2^48 + 2^47 each stay below 2^54 (40 * 1.5 = 60 < 64).  Integer
 // addition is associative, so the total does not depend on the arrival order.
 // The two flags are set with an atomic OR that precedes the contributor's add
 // (same lane, same address: performed in program order), so they are sticky and
@@ -145,7 +146,7 @@ struct Problem {
     int sets_per_split;
     int ksplit;
     float norm_eps;
-    int reserved_;
+    int twin;            // look-up kernel: 1 = the items are twin items (n_tiles counts tile pairs)
     // ---- cache line 3: needed when sums are handed over --------------------------------------
     int overwrite;       // 1: out = y instead of out += y
     // RMSNorm split over two launches (fused entry point only).  The launch that completes

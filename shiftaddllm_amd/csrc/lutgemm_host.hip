@@ -142,7 +142,7 @@ struct Option {
 constexpr Option kOptions[LUTGEMM_OPTION_COUNT] = {
     {"LUTGEMM_TARGET_BLOCKS", 0}, {"LUTGEMM_FIRST_SHARE", 60}, {"LUTGEMM_MFMA_MIN_M", 3},
     {"LUTGEMM_MFMA_BLOCKS", 0},   {"LUTGEMM_PAIR_TABLES", 1},  {"LUTGEMM_SINGLE_ITEM", 1},
-    {"LUTGEMM_CHAIN_BLOCKS", 0}, {"LUTGEMM_CHAIN_GRID", 0},
+    {"LUTGEMM_CHAIN_BLOCKS", 0}, {"LUTGEMM_CHAIN_GRID", 0},  {"LUTGEMM_TWIN_ITEMS", 4},
 };
 std::atomic<int> g_option[LUTGEMM_OPTION_COUNT];
 std::once_flag g_option_once;
@@ -189,9 +189,13 @@ int first_share()
 
 // Cut the (tile, set) items of a problem into contiguous ranges, one per workgroup,
 // aiming at `want_blocks` workgroups.
-int plan_lookup(Problem &p, int mrows, long want_blocks)
+// `twin`: the items are twin items, one set of inputs against a PAIR of output tiles (one table
+// build for 512 outputs); n_tiles counts pairs then.
+int plan_lookup(Problem &p, int mrows, long want_blocks, bool twin = false)
 {
     p.n_tiles = (p.N + kTileCols - 1) / kTileCols;
+    if (twin) p.n_tiles = (p.n_tiles + 1) / 2;
+    p.twin = twin ? 1 : 0;
     p.mchunks = (p.M + mrows - 1) / mrows;
     const long total = (long)p.n_tiles * p.nsets;
     long wgs = want_blocks / p.mchunks;
@@ -208,7 +212,14 @@ int plan_lookup(Problem &p, int mrows, long want_blocks)
     if (p.mchunks == 1 && want_blocks == 512 && total >= 2 * 256 * 2 && share > 50 && share < 100) {
         const long pair = (total + 255) / 256;
         long a = (pair * share + 99) / 100, b = pair - a;
-        if (b >= 1 && b >= cap && a > b) {
+        // (the smaller range may not fall below what the contribution count allows: give it
+        // items of the larger one while the larger one stays the larger)
+        while (b < cap && a - 1 > b + 1) {
+            --a;
+            ++b;
+        }
+        // (a split far beyond the share, 3 and 1 of 4, is worse than none: 8192x8192x4 11.4 us against 10.5)
+        if (b >= 1 && b >= cap && a > b && 100 * a <= (share + 12) * pair) {
             ipw = a;
             n_long = 256;
             short_items = b;
@@ -320,7 +331,7 @@ void plan_mfma(Problem &p, int mt, long want)
     p.nsets = p.K / kMfmaStepK;  // K-steps
     if (want > p.nsets / kMfmaWaves) want = p.nsets / kMfmaWaves;
     if (want < 1) want = 1;
-    if (want > kMaxContrib) want = kMaxContrib;
+    if (want > kMaxSlices) want = kMaxSlices;
     p.sets_per_split = (p.nsets + (int)want - 1) / (int)want;
     p.sets_per_split = (p.sets_per_split + kMfmaWaves - 1) / kMfmaWaves * kMfmaWaves;  // whole rounds
     p.ksplit = (p.nsets + p.sets_per_split - 1) / p.sets_per_split;
@@ -361,7 +372,7 @@ int mfma_slices(const Group &g, int mt)
         if (rounds > max_rounds) max_rounds = rounds;
         if (p.M > rows) rows = p.M;
     }
-    if (max_rounds > kMaxContrib) max_rounds = kMaxContrib;
+    if (max_rounds > kMaxSlices) max_rounds = kMaxSlices;
     if (const int blocks = mfma_blocks_override()) return (int)(blocks / tiles > 1 ? blocks / tiles : 1);
     if (mt != 1) return (int)(kCUs / tiles > 1 ? kCUs / tiles : 1);
     int best = 1;
@@ -449,7 +460,28 @@ int plan_single(Problem &p, int mode, int *kernel, int *mrows)
     *kernel = kLookup;
     *mrows = pick_mrows(p.M);
     const long items = (long)((p.N + kTileCols - 1) / kTileCols) * p.nsets;
-    return plan_lookup(p, *mrows, target_blocks((long)p.N * (p.K / 8) * p.nb, items, mode != kRowF16 && mode != kUniformF16));
+    const long want = target_blocks((long)p.N * (p.K / 8) * p.nb, items, mode != kRowF16 && mode != kUniformF16);
+    int rc = plan_lookup(p, *mrows, want);
+    if (rc != LUTGEMM_OK) return rc;
+    // One row, per-column alphas and ranges of several items: twin items, i.e. one table build and one
+    // barrier per 512 outputs instead of per 256.  A build is about a third of an item's vector
+    // instructions at three bit planes, and a launch whose workgroups hold several items each is bound
+    // by those; launches of one or two items per workgroup are bound by latencies that twin items would
+    // lengthen (half as many ranges to spread over the chip).
+    // Measured, plain against twin items (us): 28672x8192x4 27.2 / 24.7-25.1, 28672x8192x3 21.6 / 19.6-20.0;
+    // with two bit planes no gain (28672x8192x2 15.0 / 15.2-15.4: bound by the stream), and none where the
+    // twin plan has to give up the unequal ranges of the two workgroups of a CU (8192x28672x4 with equal
+    // ranges 26.3 / 28.1) or where K is long (the same shape with ranges of 4 and 3 twin items 26.4 / 26.9).
+    const int least = option(LUTGEMM_OPTION_TWIN_ITEMS);
+    if (least > 0 && *mrows == 1 && (mode == kRowF16 || mode == kUniformF16) && p.nb >= 3 && p.nsets <= 64 &&
+        p.short_items >= least && p.items_per_wg >= least) {
+        Problem t = p;
+        const bool unequal = p.items_per_wg != p.short_items;
+        if (plan_lookup(t, 1, want, true) == LUTGEMM_OK && (!unequal || t.items_per_wg != t.short_items) &&
+            10 * t.n_blocks >= 9 * p.n_blocks)
+            p = t;
+    }
+    return LUTGEMM_OK;
 }
 
 int run(int mode, const uint32_t *bW, const void *alpha, const void *qbias, const void *x,
@@ -1138,12 +1170,14 @@ int lutgemm_describe_plan(int format, int N, int K, int nb, int groups, int M, l
     plan->row_chunks = p.mchunks;
     if (kernel == kMatrixCore) {
         plan->tiles = p.n_tiles;
+        plan->tile_columns = kMfmaTileCols;
         plan->k_units = p.nsets;
         plan->k_slices = p.ksplit;
         plan->units_per_slice = p.sets_per_split;
         plan->needs_workspace = p.ksplit > 1;
     } else {
         plan->tiles = p.n_tiles;
+        plan->tile_columns = p.twin ? 2 * kTileCols : kTileCols;
         plan->k_units = p.nsets;
         plan->long_ranges = p.long_ranges;
         plan->items_per_long_range = p.items_per_wg;

@@ -54,7 +54,7 @@ C_ABI_SYMBOLS = (
 
 MAX_GROUP = 8
 OPTIONS = {"TARGET_BLOCKS": 0, "FIRST_SHARE": 1, "MFMA_MIN_M": 2, "MFMA_BLOCKS": 3, "PAIR_TABLES": 4, "SINGLE_ITEM": 5,
-           "CHAIN_BLOCKS": 6, "CHAIN_GRID": 7}
+           "CHAIN_BLOCKS": 6, "CHAIN_GRID": 7, "TWIN_ITEMS": 8}
 CHAIN_MAX_ROWS = 4
 CHAIN_MAX_TAG = 65534
 NOALLOC_MAX_WORDS = 1 << 18
@@ -71,7 +71,7 @@ class Plan(ctypes.Structure):
     """struct lutgemm_plan of include/lutgemm_gfx950.h."""
     _fields_ = [(n, ctypes.c_int) for n in (
         "kernel", "workgroups", "rows_per_pass", "row_chunks", "tiles", "k_units", "ranges", "long_ranges",
-        "items_per_long_range", "items_per_short_range", "k_slices", "units_per_slice", "needs_workspace")]
+        "items_per_long_range", "items_per_short_range", "k_slices", "units_per_slice", "needs_workspace", "tile_columns")]
 
 
 class FusedProblem(ctypes.Structure):

@@ -84,3 +84,33 @@ def test_every_option_setting_against_the_oracle(gpu_device, cases, name, value)
             assert rel <= 2e-4 and mad <= 1e-3, (name, value, N, K, nb, R, rel, mad)
     finally:
         lib.lutgemm_set_option(which, -1)
+
+
+def test_thirty_nine_contributions_per_output(gpu_device):
+    """One item per workgroup on a tile whose K extent is 39 sets: every output's accumulator word
+    takes 39 fixed-point contributions (the planner's limit is 40), all of one sign here so that the
+    running sum is as large as the data allows."""
+    lib = native.cabi()
+    N, K, nb = 512, 39 * 256, 2
+    g = torch.Generator().manual_seed(77)
+    bW = torch.full((K // 32, nb, N), -1, dtype=torch.int32)              # every sign +1
+    alpha = torch.full((K // 128, nb, N), 2.0 ** -6, dtype=torch.float16)
+    x = (torch.randn((1, K), generator=g).abs() * 4).half()
+    want, _ = orc.gemv_rowwise_c(bW.numpy(), alpha.numpy(), x.numpy(), K // 128)
+    which = native.OPTIONS["TARGET_BLOCKS"]
+    assert lib.lutgemm_set_option(which, 4096) == 0
+    try:
+        plan = native.Plan()
+        assert lib.lutgemm_describe_plan(0, N, K, nb, K // 128, 1, ctypes.byref(plan)) == 0
+        assert plan.items_per_long_range == 1 and plan.workgroups == 2 * 39 and plan.needs_workspace == 1
+        d = [t.to(gpu_device) for t in (bW, alpha, x)]
+        out = torch.zeros((1, N), dtype=torch.float16, device=gpu_device)
+        for _ in range(2):                                                # twice: the words must be left at zero
+            out.zero_()
+            rc = lib.lutgemm_gemv_rowwise_f16(_ptr(d[0]), _ptr(d[1]), _ptr(d[2]), _ptr(out), N, K, nb, K // 128, 1, _sp())
+            assert rc == 0, lib.lutgemm_strerror(rc).decode()
+            torch.cuda.synchronize()
+            rel, mad = orc.error_metrics(out.float().cpu().numpy(), want.astype(np.float32))
+            assert rel <= 2e-4 and mad <= 1e-3, (rel, mad)
+    finally:
+        lib.lutgemm_set_option(which, -1)

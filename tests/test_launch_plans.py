@@ -2,7 +2,7 @@
 planner's invariants are checked here over the benchmark shapes and a few thousand
 random ones.  What a kernel relies on (and cannot check itself):
   look-up kernel   the ranges cover every (tile, set) item exactly once, none is empty,
-                   and no output tile receives more than 32 contributions (the count field
+                   and no output tile receives more than 40 contributions (the count field
                    of an accumulator word, lutgemm_common.h);
   matrix cores     the K-slices cover every step, none is empty, each is a whole number of
                    eight-step rounds, and there are at most 32 of them per tile."""
@@ -14,7 +14,8 @@ import pytest
 
 LOOKUP, MATRIX_CORE = 0, 1
 ROWWISE, BLOCK_F16, BLOCK_U16, BLOCK_I8, UNIFORM = range(5)
-MAX_CONTRIB = 32
+MAX_CONTRIB = 40
+MAX_SLICES = 32
 
 
 @pytest.fixture(scope="module")
@@ -36,7 +37,9 @@ def describe(lib, fmt, N, K, nb, groups, M):
 def check_plan(p, N, K, M):
     assert p.workgroups >= 1 and p.row_chunks == -(-M // p.rows_per_pass)
     if p.kernel == LOOKUP:
-        assert p.tiles == -(-N // 256) and p.k_units == -(-K // 256)
+        assert p.tile_columns in (256, 512) and p.tiles == -(-N // p.tile_columns) and p.k_units == -(-K // 256)
+        if p.tile_columns == 512:      # twin items: one row, every range of at least two of them unless there is only one
+            assert p.rows_per_pass == 1 and M == 1
         total = p.tiles * p.k_units
         a, b, n_long, n = p.items_per_long_range, p.items_per_short_range, p.long_ranges, p.ranges
         assert a >= b >= 1 and 1 <= n_long <= n and p.workgroups == n * p.row_chunks
@@ -62,7 +65,7 @@ def check_plan(p, N, K, M):
     else:
         assert p.tiles == -(-N // 64) and p.k_units == K // 128
         assert p.rows_per_pass in (16, 32)
-        assert 1 <= p.k_slices <= MAX_CONTRIB and p.units_per_slice % 8 == 0
+        assert 1 <= p.k_slices <= MAX_SLICES and p.units_per_slice % 8 == 0
         assert p.k_slices * p.units_per_slice >= p.k_units, "slices must cover every K-step"
         assert (p.k_slices - 1) * p.units_per_slice < p.k_units, "no slice may be empty"
         assert p.workgroups == p.tiles * p.k_slices * p.row_chunks
