@@ -96,6 +96,31 @@ int lutgemm_gemv_rowwise_f16(const uint32_t *bW, const void *alpha_f16, const vo
                              void *stream);
 
 /*
+ * lutgemm_gemv_rowwise_f16 for alphas that are POWERS OF TWO, which is what ShiftAddLLM's
+ * quantiser produces (quantizers/bcq_quant/bcq_shift.py:15-24,34: every alpha is rounded
+ * to 2^round(log2 |alpha|)) and what gives the method its name: multiplying by such an
+ * alpha is a shift.  Same arguments and semantics; the caller PROMISES that every alpha
+ * is a positive normal fp16 power of two (mantissa bits zero, exponent field 1..30).
+ * With that promise and three or more rows (M >= 3, K a multiple of 128, groups of a
+ * multiple of 128 inputs, N a multiple of 16) the call runs on gfx950's block-scaled matrix
+ * instruction: sign bits become 4-bit floats +-1 through a table (one LDS read per eight
+ * signs), the alpha's exponent rides as the instruction's per-block power-of-two scale, and
+ * the activations are split, by a small kernel in front, into three 8-bit floats per value
+ * with a power-of-two scale per 32 (exact for every fp16 value within 2^14 of the largest
+ * of its 32; smaller ones are cut off at 2^-25 of it).  Accumulation is fp32, one rounding
+ * to fp16 at the end, as in every other entry point.  An infinity or NaN among the
+ * activations gives NaN in every output of its row.  Other calls (fewer rows, other shapes)
+ * run exactly as lutgemm_gemv_rowwise_f16 does.  With an alpha that breaks the promise the
+ * result is that of the alpha with its mantissa bits cleared (zero counts as 2^-15).
+ * The split activations (3 * M * K + M * K / 8 bytes) live in a second per-stream buffer
+ * that grows like the accumulator workspace: make one call of each size before capturing
+ * a graph.  No counterpart in the reference.
+ */
+int lutgemm_gemv_rowwise_pow2_f16(const uint32_t *bW, const void *alpha_f16, const void *x_f16,
+                                  void *out_f16, int N, int K, int nb, int num_groups, int M,
+                                  void *stream);
+
+/*
  * lutgemm_gemv_rowwise_f16 for callers that cannot allocate device memory: code
  * under HIP graph capture, tight serving loops, harnesses that forbid it.  It
  * has no counterpart in the reference.  Same arguments, semantics and results,
@@ -231,7 +256,7 @@ int lutgemm_reserve_workspace(void *stream, size_t words);
 #define LUTGEMM_FORMAT_UNIFORM_F16 4
 
 typedef struct lutgemm_plan {
-    int kernel;          /* 0: table look-up kernel, 1: matrix-core kernel */
+    int kernel;          /* 0: table look-up kernel, 1: matrix-core kernel, 2: block-scaled matrix-core kernel */
     int workgroups;      /* of the launch */
     int rows_per_pass;   /* activation rows a workgroup handles together */
     int row_chunks;      /* ceil(M / rows_per_pass) */
@@ -249,6 +274,10 @@ typedef struct lutgemm_plan {
 } lutgemm_plan;
 
 int lutgemm_describe_plan(int format, int N, int K, int nb, int groups, int M, lutgemm_plan *plan);
+/* The same for lutgemm_gemv_rowwise_pow2_f16: kernel 2 is the block-scaled matrix-core kernel
+ * (rows_per_pass 5, 8 or 16; tiles of 64 columns, steps of 128 inputs); a call that takes one
+ * of the other kernels is described as lutgemm_describe_plan describes it. */
+int lutgemm_describe_pow2_plan(int N, int K, int nb, int groups, int M, lutgemm_plan *plan);
 
 /*
  * Tuning options (no counterpart in the reference, whose launch geometry is fixed at
@@ -271,6 +300,10 @@ int lutgemm_describe_plan(int format, int N, int K, int nb, int groups, int M, l
  *   TWIN_ITEMS    : one-row look-up launches whose workgroups would all hold at least this
  *                   many items take twin items instead (one table build per 512 outputs
  *                   instead of per 256; default 4, 0 = never)
+ *   BLOCK_SCALED  : lutgemm_gemv_rowwise_pow2_f16 takes the block-scaled matrix-core
+ *                   kernel 1 = where it is the faster one (few rows, large matrices),
+ *                   2 = wherever it applies, 0 = never (the call then behaves like
+ *                   lutgemm_gemv_rowwise_f16); default 1
  *   CHAIN_GRID    : workgroups of a chained launch (0 = as many as the device holds
  *                   at once, which is also the upper limit)
  *   CHAIN_BLOCKS  : ranges the problems of one stage of a chained launch are cut into
@@ -285,7 +318,8 @@ int lutgemm_describe_plan(int format, int N, int K, int nb, int groups, int M, l
 #define LUTGEMM_OPTION_CHAIN_BLOCKS 6
 #define LUTGEMM_OPTION_CHAIN_GRID 7
 #define LUTGEMM_OPTION_TWIN_ITEMS 8
-#define LUTGEMM_OPTION_COUNT 9
+#define LUTGEMM_OPTION_BLOCK_SCALED 9
+#define LUTGEMM_OPTION_COUNT 10
 int lutgemm_set_option(int which, int value);
 int lutgemm_get_option(int which);
 

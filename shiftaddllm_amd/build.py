@@ -49,9 +49,9 @@ def _run(cmd):
 
 
 KERNEL_SOURCES = ("lutgemm_host.hip", "lut_gemv_rowwise.hip", "lut_gemv_block.hip", "lut_gemv_block_staged.hip",
-                  "lut_gemv_group.hip", "lut_gemv_fused.hip", "lut_gemv_chain.hip", "lut_gemm_mfma.hip", "decode_kernels.hip")
+                  "lut_gemv_group.hip", "lut_gemv_fused.hip", "lut_gemv_chain.hip", "lut_gemm_mfma.hip", "lut_gemm_mx.hip", "decode_kernels.hip")
 KERNEL_HEADERS = ("lutgemm_internal.h", "lutgemm_common.h", "lutgemm_launch.h", "lut_gemv_device.h",
-                  "lut_gemm_mfma_device.h")
+                  "lut_gemm_mfma_device.h", "lut_gemm_mx_device.h")
 
 
 def build_kernel_library(force: bool = False, timestamps: bool = False) -> str:

@@ -72,6 +72,10 @@ struct Workspace {
     unsigned long long *accum = nullptr;
     size_t words = 0;
     std::vector<unsigned long long *> retired;  // outgrown buffers: captured graphs may still name them
+    // second buffer of the block-scaled matrix-core path: the split activations of the call in flight
+    void *split = nullptr;
+    size_t split_bytes = 0;
+    std::vector<void *> retired_split;
 };
 
 std::mutex g_ws_mutex;
@@ -115,6 +119,37 @@ int stream_workspace(hipStream_t stream, size_t words, unsigned long long **out)
     return LUTGEMM_OK;
 }
 
+// The same for the split activations of the block-scaled path (not zeroed: every call writes what it
+// reads).  Calls on one stream are ordered, so they can share the buffer.
+int stream_split_buffer(hipStream_t stream, size_t bytes, void **out)
+{
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return hip_fail(e);
+    std::lock_guard<std::mutex> lock(g_ws_mutex);
+    Workspace &ws = g_workspaces[std::make_pair(dev, stream)];
+    if (ws.split_bytes < bytes) {
+        hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+        e = hipStreamIsCapturing(stream, &cap);
+        if (e != hipSuccess) return hip_fail(e);
+        if (cap != hipStreamCaptureStatusNone) return LUTGEMM_ECAPTURE;
+        e = hipStreamSynchronize(stream);
+        if (e != hipSuccess) return hip_fail(e);
+        if (ws.split) ws.retired_split.push_back(ws.split);
+        ws.split = nullptr;
+        ws.split_bytes = 0;
+        const size_t want = bytes < (1u << 20) ? (1u << 20) : bytes;
+        e = hipMalloc(&ws.split, want);
+        if (e != hipSuccess) {
+            g_last_hip_error = (int)e;
+            return LUTGEMM_ENOMEM;
+        }
+        ws.split_bytes = want;
+    }
+    *out = ws.split;
+    return LUTGEMM_OK;
+}
+
 // Where a call takes its accumulator words from.
 struct Accum {
     hipStream_t stream;
@@ -143,6 +178,7 @@ constexpr Option kOptions[LUTGEMM_OPTION_COUNT] = {
     {"LUTGEMM_TARGET_BLOCKS", 0}, {"LUTGEMM_FIRST_SHARE", 60}, {"LUTGEMM_MFMA_MIN_M", 3},
     {"LUTGEMM_MFMA_BLOCKS", 0},   {"LUTGEMM_PAIR_TABLES", 1},  {"LUTGEMM_SINGLE_ITEM", 1},
     {"LUTGEMM_CHAIN_BLOCKS", 0}, {"LUTGEMM_CHAIN_GRID", 0},  {"LUTGEMM_TWIN_ITEMS", 4},
+    {"LUTGEMM_BLOCK_SCALED", 1},
 };
 std::atomic<int> g_option[LUTGEMM_OPTION_COUNT];
 std::once_flag g_option_once;
@@ -484,12 +520,85 @@ int plan_single(Problem &p, int mode, int *kernel, int *mrows)
     return LUTGEMM_OK;
 }
 
+// Block-scaled kernel: a workgroup takes 64 outputs, a chunk of 5, 8 or 16 rows and a K-slice of whole rounds (8 K-steps,
+// one per wave); two workgroups fit a CU.  The slice length (rounds) is the one that minimises the
+// rounds of the grid times the cost of a workgroup: its rounds plus a constant for its start and end
+// (table build, reduction, accumulator words), in units of a round.
+void plan_mx(Problem &p)
+{
+    constexpr long kResident = 2 * 256;
+    // (measured: anything from half a round to three rounds plans the same launches for the shapes
+    // tried; with no constant at all a slice is a single round and 28672x8192x4 takes 61 us instead of 34)
+    constexpr double fixed_rounds = 1.0;
+    p.n_tiles = (p.N + kMfmaTileCols - 1) / kMfmaTileCols;
+    p.mchunks = (p.M + mx_chunk_rows(p.M) - 1) / mx_chunk_rows(p.M);
+    p.nsets = p.K / kMfmaStepK;
+    const int rounds = (p.nsets + kMfmaWaves - 1) / kMfmaWaves;
+    int best = rounds;
+    double best_cost = 0.0;
+    for (int r = rounds; r >= 1; --r) {
+        const int ks = (rounds + r - 1) / r;
+        if (ks > kMaxSlices) break;
+        const long wgs = (long)p.n_tiles * p.mchunks * ks;
+        const double cost = (double)((wgs + kResident - 1) / kResident) * ((double)r + fixed_rounds);
+        if (r == rounds || cost < best_cost * 0.999) {
+            best = r;
+            best_cost = cost;
+        }
+    }
+    if (const int blocks = mfma_blocks_override()) {
+        long want = blocks / ((long)p.n_tiles * p.mchunks);
+        if (want < 1) want = 1;
+        if (want > kMaxSlices) want = kMaxSlices;
+        if (want > rounds) want = rounds;
+        best = (rounds + (int)want - 1) / (int)want;
+    }
+    p.sets_per_split = best * kMfmaWaves;
+    p.ksplit = (p.nsets + p.sets_per_split - 1) / p.sets_per_split;
+    p.n_blocks = p.n_tiles * p.ksplit * p.mchunks;
+}
+
+// Whether a problem that may take the block-scaled kernel should.  It needs one, two or three matrix
+// instructions per (bit plane, 16 outputs, 128 inputs) for up to 5, 8 or 16 rows where the fp16 kernel
+// needs four (and its sign expansion), but also a launch of its own that splits the activations
+// (3 to 4 us with the gap between the launches).  Measured (us, fp16 kernel vs block-scaled):
+//   28672x8192x4: 4 rows 50.8 / 33.5, 8 rows 50.1 / 40.2, 16 rows 48.4 / 58.3
+//   28672x8192x2: 4 rows 27.1 / 23.5, 8 rows 29.0 / 30.2
+//   8192x8192x4:  4 rows 17.0 / 16.4, 8 rows 17.8 / 18.6;  8192x8192x2: 4 rows 11.2 / 13.6
+// so: up to 5 rows from 48 MB of sign words on, up to 8 rows from 96 MB on.
+bool mx_wanted(const Problem &p)
+{
+    const int how = option(LUTGEMM_OPTION_BLOCK_SCALED);
+    if (how != 1) return how == 2;
+    const long sign_bytes = (long)p.N * (p.K / 8) * p.nb;
+    return (p.M <= 5 && sign_bytes >= (48l << 20)) || (p.M <= 8 && sign_bytes >= (96l << 20));
+}
+
+// Row-wise problem whose alphas are powers of two, with enough rows for the matrix cores: the
+// block-scaled kernel (16-row tiles; more rows are further row chunks that stream the same sign
+// words side by side).
+int run_mx(Problem &p, const Accum &acc)
+{
+    plan_mx(p);
+    if (p.ksplit > 1) {
+        int rc = accum_words(acc, (size_t)p.M * p.N, &p.accum);
+        if (rc != LUTGEMM_OK) return rc;
+    }
+    if (acc.fixed) return LUTGEMM_EUNSUP;
+    void *buf = nullptr;
+    int rc = stream_split_buffer(acc.stream, mx_split_bytes(p.M, p.K), &buf);
+    if (rc != LUTGEMM_OK) return rc;
+    const hipError_t e = launch_mx(p, buf, acc.stream);
+    return e == hipSuccess ? LUTGEMM_OK : hip_fail(e);
+}
+
 int run(int mode, const uint32_t *bW, const void *alpha, const void *qbias, const void *x,
-        void *out, int N, int K, int nb, int num_groups, int M, const Accum &acc)
+        void *out, int N, int K, int nb, int num_groups, int M, const Accum &acc, bool alpha_pow2 = false)
 {
     Problem p;
     int rc = fill_problem(p, mode, bW, alpha, qbias, x, out, N, K, nb, num_groups, M);
     if (rc != LUTGEMM_OK) return rc;
+    if (alpha_pow2 && mode == kRowF16 && mfma_eligible(p, mode) && p.M >= mfma_min_rows() && mx_wanted(p)) return run_mx(p, acc);
     int kernel = kLookup, mrows = 1;
     rc = plan_single(p, mode, &kernel, &mrows);
     if (rc != LUTGEMM_OK) return rc;
@@ -992,6 +1101,14 @@ int lutgemm_gemv_rowwise_f16(const uint32_t *bW, const void *alpha_f16, const vo
                Accum{(hipStream_t)stream});
 }
 
+int lutgemm_gemv_rowwise_pow2_f16(const uint32_t *bW, const void *alpha_f16, const void *x_f16,
+                                  void *out_f16, int N, int K, int nb, int num_groups, int M,
+                                  void *stream)
+{
+    return run(kRowF16, bW, alpha_f16, nullptr, x_f16, out_f16, N, K, nb, num_groups, M,
+               Accum{(hipStream_t)stream}, true);
+}
+
 int lutgemm_gemv_rowwise_f16_noalloc(const uint32_t *bW, const void *alpha_f16, const void *x_f16,
                                      void *out_f16, int N, int K, int nb, int num_groups, int M,
                                      void *stream)
@@ -1188,6 +1305,30 @@ int lutgemm_describe_plan(int format, int N, int K, int nb, int groups, int M, l
     return LUTGEMM_OK;
 }
 
+int lutgemm_describe_pow2_plan(int N, int K, int nb, int groups, int M, lutgemm_plan *plan)
+{
+    int rc = lutgemm_describe_plan(LUTGEMM_FORMAT_ROWWISE_F16, N, K, nb, groups, M, plan);
+    if (rc != LUTGEMM_OK) return rc;
+    alignas(16) static const uint64_t dummy[2] = {0, 0};
+    Problem p;
+    rc = fill_problem(p, kRowF16, (const uint32_t *)dummy, dummy, dummy, dummy, (void *)dummy, N, K, nb, groups, M);
+    if (rc != LUTGEMM_OK) return rc;
+    if (!(mfma_eligible(p, kRowF16) && p.M >= mfma_min_rows() && mx_wanted(p))) return LUTGEMM_OK;
+    plan_mx(p);
+    *plan = lutgemm_plan{};
+    plan->kernel = 2;
+    plan->workgroups = p.n_blocks;
+    plan->rows_per_pass = mx_chunk_rows(p.M);
+    plan->row_chunks = p.mchunks;
+    plan->tiles = p.n_tiles;
+    plan->tile_columns = kMfmaTileCols;
+    plan->k_units = p.nsets;
+    plan->k_slices = p.ksplit;
+    plan->units_per_slice = p.sets_per_split;
+    plan->needs_workspace = p.ksplit > 1;
+    return LUTGEMM_OK;
+}
+
 size_t lutgemm_workspace_words(int N, int M)
 {
     if (N <= 0 || M <= 0) return 0;
@@ -1252,6 +1393,8 @@ int lutgemm_release_workspaces(void)
         if (it->first.first == dev) {
             if (it->second.accum) (void)hipFree(it->second.accum);
             for (unsigned long long *old : it->second.retired) (void)hipFree(old);
+            if (it->second.split) (void)hipFree(it->second.split);
+            for (void *old : it->second.retired_split) (void)hipFree(old);
             it = g_workspaces.erase(it);
         } else {
             ++it;

@@ -27,6 +27,12 @@ hipError_t chain_resident_workgroups(int *count);
 hipError_t launch_mfma(const Problem &p, int mt, hipStream_t stream);
 hipError_t launch_mfma_fused(const Problem &p, int mt, hipStream_t stream);  // one problem with fused extras
 hipError_t launch_mfma_group(const Group &g, int mt, int blocks, hipStream_t stream);
+// block-scaled matrix-core kernel (alphas are powers of two): splits p.x into `split` (mx_split_bytes:
+// three pieces per value, a row of zeros, a scale word per block of 32), then runs the problem; grid =
+// p.n_blocks, row chunks of mx_chunk_rows(p.M) rows
+hipError_t launch_mx(const Problem &p, void *split, hipStream_t stream);
+inline int mx_chunk_rows(int M) { return M <= 5 ? 5 : M <= 8 ? 8 : 16; }
+inline size_t mx_split_bytes(int M, int K) { return (size_t)M * K * 3 + (size_t)K + (size_t)M * (K / 32) * 4; }
 
 }  // namespace lutgemm
 

@@ -22,6 +22,7 @@ C_ABI_SYMBOLS = (
     "lutgemm_strerror",
     "lutgemm_last_hip_error",
     "lutgemm_gemv_rowwise_f16",
+    "lutgemm_gemv_rowwise_pow2_f16",
     "lutgemm_gemv_rowwise_f16_noalloc",
     "lutgemm_gemv_rowwise_f16_grouped",
     "lutgemm_gemv_rowwise_f16_fused",
@@ -40,6 +41,7 @@ C_ABI_SYMBOLS = (
     "lutgemm_workspace_words",
     "lutgemm_reserve_workspace",
     "lutgemm_describe_plan",
+    "lutgemm_describe_pow2_plan",
     "lutgemm_set_option",
     "lutgemm_set_timestamp_buffer",
     "lutgemm_get_option",
@@ -54,7 +56,7 @@ C_ABI_SYMBOLS = (
 
 MAX_GROUP = 8
 OPTIONS = {"TARGET_BLOCKS": 0, "FIRST_SHARE": 1, "MFMA_MIN_M": 2, "MFMA_BLOCKS": 3, "PAIR_TABLES": 4, "SINGLE_ITEM": 5,
-           "CHAIN_BLOCKS": 6, "CHAIN_GRID": 7, "TWIN_ITEMS": 8}
+           "CHAIN_BLOCKS": 6, "CHAIN_GRID": 7, "TWIN_ITEMS": 8, "BLOCK_SCALED": 9}
 CHAIN_MAX_ROWS = 4
 CHAIN_MAX_TAG = 65534
 NOALLOC_MAX_WORDS = 1 << 18
@@ -136,6 +138,8 @@ def _bind(lib: ctypes.CDLL) -> ctypes.CDLL:
     lib.lutgemm_last_hip_error.argtypes = []
     lib.lutgemm_last_hip_error.restype = ci
     lib.lutgemm_gemv_rowwise_f16.argtypes = [vp, vp, vp, vp, ci, ci, ci, ci, ci, vp]
+    lib.lutgemm_gemv_rowwise_pow2_f16.argtypes = [vp, vp, vp, vp, ci, ci, ci, ci, ci, vp]
+    lib.lutgemm_gemv_rowwise_pow2_f16.restype = ci
     lib.lutgemm_gemv_rowwise_f16_noalloc.argtypes = [vp, vp, vp, vp, ci, ci, ci, ci, ci, vp]
     lib.lutgemm_gemv_rowwise_f16_noalloc.restype = ci
     lib.lutgemm_gemv_rowwise_f16_grouped.argtypes = [ci, ctypes.POINTER(RowwiseProblem), vp]
@@ -167,6 +171,8 @@ def _bind(lib: ctypes.CDLL) -> ctypes.CDLL:
     lib.lutgemm_copy_bytes.restype = ci
     lib.lutgemm_describe_plan.argtypes = [ci, ci, ci, ci, ci, ci, ctypes.POINTER(Plan)]
     lib.lutgemm_describe_plan.restype = ci
+    lib.lutgemm_describe_pow2_plan.argtypes = [ci, ci, ci, ci, ci, ctypes.POINTER(Plan)]
+    lib.lutgemm_describe_pow2_plan.restype = ci
     lib.lutgemm_set_option.argtypes = [ci, ci]
     lib.lutgemm_set_option.restype = ci
     lib.lutgemm_get_option.argtypes = [ci]

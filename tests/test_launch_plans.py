@@ -282,3 +282,46 @@ def test_chain_plan_validation_on_the_host(lib):
     # units of more than sixteen items would not fit one activation window: the stage takes more rounds
     rc, plan = _describe_chain(lib, [_chain_problem(A, 8192, 8192, 3, x, o)], 8)
     assert rc == 0 and plan.workgroups == 8 and plan.items_per_unit[0] <= 16 and plan.unit_count[0] >= 64
+
+
+def test_pow2_plan_takes_the_block_scaled_kernel_for_few_rows_of_large_matrices():
+    """lutgemm_describe_pow2_plan: up to 5 rows from 48 MB of sign words on and up to 8 rows from 96 MB
+    on run block-scaled (kernel 2) in chunks of 5 or 8 rows; everything else is planned as
+    lutgemm_gemv_rowwise_f16 plans it.  Option BLOCK_SCALED: 0 never, 2 wherever the kernel applies."""
+    import ctypes
+    from shiftaddllm_amd import native
+    lib = native.cabi()
+    which = native.OPTIONS["BLOCK_SCALED"]
+
+    def plan(N, K, nb, M, group=128):
+        p = native.Plan()
+        assert lib.lutgemm_describe_pow2_plan(N, K, nb, K // group, M, ctypes.byref(p)) == 0
+        return p
+
+    def same_as_fp16(N, K, nb, M, group=128):
+        a, b = plan(N, K, nb, M, group), native.Plan()
+        assert lib.lutgemm_describe_plan(0, N, K, nb, K // group, M, ctypes.byref(b)) == 0
+        return bytes(a) == bytes(b)
+
+    try:
+        lib.lutgemm_set_option(which, 1)
+        p = plan(28672, 8192, 4, 4)
+        assert (p.kernel, p.rows_per_pass, p.row_chunks, p.tile_columns, p.tiles) == (2, 5, 1, 64, 448)
+        assert p.k_units == 64 and p.k_slices * p.units_per_slice >= 64 and p.workgroups == 448 * p.k_slices
+        assert p.needs_workspace == (p.k_slices > 1)
+        assert plan(28672, 8192, 2, 5).kernel == 2            # 56 MB
+        p = plan(28672, 8192, 4, 8)                           # 112 MB
+        assert (p.kernel, p.rows_per_pass) == (2, 8)
+        assert same_as_fp16(28672, 8192, 2, 8)                # 8 rows want 96 MB
+        assert same_as_fp16(28672, 8192, 4, 16)               # more than 8 rows: the fp16 kernel
+        assert same_as_fp16(4096, 4096, 3, 4)                 # small matrix
+        assert same_as_fp16(28672, 8192, 4, 1) and same_as_fp16(28672, 8192, 4, 2)   # look-up kernel
+        assert same_as_fp16(28672, 8192, 4, 4, group=32)      # groups of 32: not a matrix-core shape
+        lib.lutgemm_set_option(which, 2)
+        p = plan(4096, 4096, 3, 33)
+        assert (p.kernel, p.rows_per_pass, p.row_chunks) == (2, 16, 3)
+        assert same_as_fp16(4096, 4096, 3, 2)
+        lib.lutgemm_set_option(which, 0)
+        assert same_as_fp16(28672, 8192, 4, 4)
+    finally:
+        lib.lutgemm_set_option(which, -1)
