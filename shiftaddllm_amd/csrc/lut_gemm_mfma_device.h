@@ -52,12 +52,14 @@ constexpr int kMfmaRedBytes = kMfmaWaves * 16 * MT * kRedRow * 4;
 template <int MT>
 constexpr int kMfmaLdsBytes = kMfmaRedBytes<MT> + 16 * MT * 4;
 
-// Operands of one K-step of a wave: per bit plane word kb of 4 outputs and their
-// alphas; per 16-row tile the lane's 32 activations.
+// Operands of one K-step of a wave: per bit plane word kb of 4 outputs; the alphas of
+// those 4 outputs for bit plane kb (one load covers all planes: lane group kb of the wave
+// takes plane kb, and hands them to the other groups by lane permutes when the plane's
+// turn comes); per 16-row tile the lane's 32 activations.
 template <int NB, int MT>
 struct MfmaOperands {
     u32x4 w[NB];
-    u32x2 alpha[NB];
+    u32x2 alpha;
     u32x4 x[MT][4];
 };
 
@@ -77,8 +79,7 @@ __device__ __forceinline__ void mfma_load(MfmaOperands<NB, MT> &r, const Problem
         for (int c = 0; c < 4; ++c) r.x[mt][c] = *(const u32x4 *)(xlane[mt] + step * kMfmaStepK + 8 * c);
     const int g = fast_div(step * 4, p.by_group_words);
     const char *abase = (const char *)p.alpha + (size_t)g * NB * (p.N * 2u) + (wcol4 >> 1);
-#pragma unroll
-    for (int b = 0; b < NB; ++b) r.alpha[b] = *(const u32x2 *)(abase + (size_t)b * (p.N * 2u));
+    r.alpha = *(const u32x2 *)(abase + (size_t)min(kb, NB - 1) * (p.N * 2u));
 }
 
 // 8 signs of sign word `w` -> 8 fp16 values +-alpha (bit set = +alpha): pair i holds
@@ -177,7 +178,9 @@ __device__ __forceinline__ void mfma_tile(const Problem &p, int local_block, cha
 #pragma unroll
         for (int b = 0; b < NB; ++b) {
             const uint32_t w4[4] = {ops.w[b].x, ops.w[b].y, ops.w[b].z, ops.w[b].w};
-            const u32x2 al = ops.alpha[b];
+            const int from = 4 * (16 * b + li);   // the lane of group b that holds this lane's outputs
+            const u32x2 al = {(uint32_t)__builtin_amdgcn_ds_bpermute(from, (int)ops.alpha.x),
+                              (uint32_t)__builtin_amdgcn_ds_bpermute(from, (int)ops.alpha.y)};
             // the alpha of output e in both halves of a register
             const uint32_t a2[4] = {__builtin_amdgcn_perm(al.x, al.x, 0x01000100u), __builtin_amdgcn_perm(al.x, al.x, 0x03020302u),
                                     __builtin_amdgcn_perm(al.y, al.y, 0x01000100u), __builtin_amdgcn_perm(al.y, al.y, 0x03020302u)};

@@ -220,7 +220,8 @@ __device__ __forceinline__ void mx_tile(const Problem &p, const MxActivations &a
         uint32_t *lut = (uint32_t *)xs;
 #pragma unroll 4
         for (int idx = tid; idx < kMxLutBytes / 4; idx += kMfmaThreads) {   // a wave writes one entry's 64 copies
-            uint32_t v = (uint32_t)(idx >> 6);          // bit j of the entry index -> bit 4 * j + 3
+            // (the entry index is the same for the whole wave: scalar arithmetic)
+            uint32_t v = (uint32_t)__builtin_amdgcn_readfirstlane(idx >> 6);   // bit j of it -> bit 4 * j + 3
             v = (v | (v << 12)) & 0x000f000fu;
             v = (v | (v << 6)) & 0x03030303u;
             v = (v | (v << 3)) & 0x11111111u;
