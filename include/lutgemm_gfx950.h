@@ -101,20 +101,23 @@ int lutgemm_gemv_rowwise_f16(const uint32_t *bW, const void *alpha_f16, const vo
  * to 2^round(log2 |alpha|)) and what gives the method its name: multiplying by such an
  * alpha is a shift.  Same arguments and semantics; the caller PROMISES that every alpha
  * is a positive normal fp16 power of two (mantissa bits zero, exponent field 1..30).
- * With that promise and three or more rows (M >= 3, K a multiple of 128, groups of a
- * multiple of 128 inputs, N a multiple of 16) the call runs on gfx950's block-scaled matrix
- * instruction: sign bits become 4-bit floats +-1 through a table (one LDS read per eight
- * signs), the alpha's exponent rides as the instruction's per-block power-of-two scale, and
- * the activations are split, by a small kernel in front, into three 8-bit floats per value
- * with a power-of-two scale per 32 (exact for every fp16 value within 2^14 of the largest
- * of its 32; smaller ones are cut off at 2^-25 of it).  Accumulation is fp32, one rounding
- * to fp16 at the end, as in every other entry point.  An infinity or NaN among the
- * activations gives NaN in every output of its row.  Other calls (fewer rows, other shapes)
- * run exactly as lutgemm_gemv_rowwise_f16 does.  With an alpha that breaks the promise the
- * result is that of the alpha with its mantissa bits cleared (zero counts as 2^-15).
- * The split activations (3 * M * K + M * K / 8 bytes) live in a second per-stream buffer
- * that grows like the accumulator workspace: make one call of each size before capturing
- * a graph.  No counterpart in the reference.
+ * With that promise a call of 3 to 8 rows on a large matrix (K a multiple of 128, groups of a
+ * multiple of 128 inputs, N a multiple of 16; up to 5 rows from 48 MB of sign words on, up
+ * to 8 rows from 96 MB on; option LUTGEMM_OPTION_BLOCK_SCALED widens or switches off the
+ * rule, lutgemm_describe_pow2_plan tells what a call takes) runs on gfx950's block-scaled
+ * matrix instruction: sign bits become 4-bit floats +-1 through a table (one LDS read per
+ * eight signs), the alpha's exponent rides as the instruction's per-block power-of-two
+ * scale, and the activations are split, by a small kernel in front, into three 8-bit floats
+ * per value with a power-of-two scale per 32 (exact for every fp16 value within 2^14 of the
+ * largest of its 32; smaller ones are cut off at 2^-25 of it); the three pieces of up to
+ * 5 rows share the 16 columns of one instruction.  Accumulation is fp32, one rounding to
+ * fp16 at the end, as in every other entry point.  An infinity or NaN among the activations
+ * gives NaN in every output of its row.  Other calls run exactly as
+ * lutgemm_gemv_rowwise_f16 does.  With an alpha that breaks the promise the result is that
+ * of the alpha with its mantissa bits cleared (zero counts as 2^-15).
+ * The split activations (3 * M * K + K + M * K / 8 bytes) live in a second per-stream
+ * buffer that grows like the accumulator workspace: make one call of each size before
+ * capturing a graph.  No counterpart in the reference.
  */
 int lutgemm_gemv_rowwise_pow2_f16(const uint32_t *bW, const void *alpha_f16, const void *x_f16,
                                   void *out_f16, int N, int K, int nb, int num_groups, int M,

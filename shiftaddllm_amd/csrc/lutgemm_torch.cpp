@@ -87,6 +87,25 @@ void lutgemm_compute_shift_scale(torch::Tensor output, torch::Tensor bWeight, to
     raise_on_error(rc, "lutgemm_compute_shift_scale");
 }
 
+// lutgemm_compute_shift_scale for alphas the caller knows to be powers of two (what the
+// reference's quantiser produces, quantizers/bcq_quant/bcq_shift.py:15-24): a few rows on a large
+// matrix take the block-scaled matrix-core kernel.  No counterpart in the reference's extension.
+void lutgemm_compute_shift_scale_pow2(torch::Tensor output, torch::Tensor bWeight, torch::Tensor alpha,
+                                      torch::Tensor d_input, int64_t mSize, int64_t kSize, int64_t nb,
+                                      int64_t num_groups)
+{
+    check_common(output, bWeight, d_input, mSize, kSize, nb);
+    TORCH_CHECK(num_groups > 0 && kSize % num_groups == 0 && (kSize / num_groups) % 32 == 0,
+                "kSize/num_groups must be a multiple of 32");
+    check_alpha(alpha, output, torch::kHalf, num_groups * nb * mSize, "alpha [num_groups, nb, mSize]");
+    const c10::hip::HIPGuardMasqueradingAsCUDA guard(output.device());
+    int rc = lutgemm_gemv_rowwise_pow2_f16((const uint32_t *)bWeight.data_ptr<int32_t>(), alpha.data_ptr(),
+                                           d_input.data_ptr(), output.data_ptr(), (int)mSize, (int)kSize,
+                                           (int)nb, (int)num_groups, rows_of(d_input, kSize),
+                                           c10::hip::getCurrentHIPStreamMasqueradingAsCUDA().stream());
+    raise_on_error(rc, "lutgemm_compute_shift_scale_pow2");
+}
+
 // lutgemm_cuda.cpp:88-98
 void lutgemm_compute(torch::Tensor output, torch::Tensor bWeight, torch::Tensor alpha,
                      torch::Tensor q_bias, torch::Tensor d_input, int64_t mSize, int64_t kSize,
@@ -280,6 +299,8 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m)
     m.doc() = "MI355X (gfx950) LUT-GEMM engine behind the ShiftAddLLM `lutgemm` call signatures";
     m.def("lutgemm_compute", &lutgemm_compute, "uniform-quant LUT-GEMV (alpha, q_bias)");
     m.def("lutgemm_compute_shift_scale", &lutgemm_compute_shift_scale, "row-wise alpha LUT-GEMV");
+    m.def("lutgemm_compute_shift_scale_pow2", &lutgemm_compute_shift_scale_pow2,
+          "row-wise alpha LUT-GEMV, alphas promised to be powers of two");
     m.def("lutgemm_compute_block", &lutgemm_compute_block, "block alpha LUT-GEMV (fp16 alpha)");
     m.def("lutgemm_compute_block_shift", &lutgemm_compute_block_shift,
           "block alpha LUT-GEMV (uint16 shift fields)");

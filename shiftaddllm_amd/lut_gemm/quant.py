@@ -108,6 +108,7 @@ class LutLinear(nn.Module):
         # kept as a plain attribute like the reference (quant.py:28)
         self.bias = bias
         self.reuse_output = False      # see _output
+        self._pow2_cache = None        # see _alphas_are_powers_of_two
         self._bias_cache = None
         self._out_cache = {}
 
@@ -134,6 +135,20 @@ class LutLinear(nn.Module):
             t = b.detach().to(device=device, dtype=torch.float16).reshape(1, self.N).expand(rows, self.N).contiguous()
             self._bias_cache = (key, t)
         return self._bias_cache[1]
+
+    def _alphas_are_powers_of_two(self):
+        """Whether every row-wise alpha is a positive normal fp16 power of two (what the reference's
+        quantiser produces, quantizers/bcq_quant/bcq_shift.py:15-24): looked at once per state of the
+        alpha tensor (one device synchronisation), and only by calls of three or more rows, which
+        can then take the block-scaled matrix-core kernel."""
+        a = self.alpha
+        key = (a.data_ptr(), a._version, a.device)
+        if self._pow2_cache is None or self._pow2_cache[0] != key:
+            bits = a.view(torch.int16).to(torch.int32) & 0xffff
+            field = (bits >> 10) & 0x1f
+            ok = ((bits & 0x83ff) == 0) & (field >= 1) & (field <= 30)
+            self._pow2_cache = (key, bool(ok.all().item()))
+        return self._pow2_cache[1]
 
     def _output(self, rows, device):
         """The tensor the kernel accumulates into, pre-filled with the bias (or zeros): a new
@@ -177,6 +192,9 @@ class LutLinear(nn.Module):
         elif fmt == "block_shift_u16":
             ext.lutgemm_compute_block_shift(output, self.binaryWeight, self.alpha, x2, self.N,
                                             self.K, self.wbit, self.num_groups, 3)
+        elif 3 <= x2.shape[0] <= 8 and self._alphas_are_powers_of_two():
+            ext.lutgemm_compute_shift_scale_pow2(output, self.binaryWeight, self.alpha, x2, self.N,
+                                                 self.K, self.wbit, self.num_groups)
         else:
             ext.lutgemm_compute_shift_scale(output, self.binaryWeight, self.alpha, x2, self.N,
                                             self.K, self.wbit, self.num_groups)

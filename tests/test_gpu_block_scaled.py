@@ -133,3 +133,36 @@ def test_default_rule_takes_the_block_scaled_kernel_for_few_rows_of_a_large_matr
         got = _run(lib.lutgemm_gemv_rowwise_pow2_f16, gpu_device, bW, alpha, x, bias)
         rel, mad = orc.error_metrics(got.float().cpu().numpy(), want.astype(np.float32))
         assert rel <= 2e-4 and mad <= 1e-3, (M, rel, mad)
+
+
+def test_lutlinear_takes_the_pow2_entry_for_a_few_rows(gpu_device):
+    """LutLinear.forward looks at its alphas once: powers of two and 3 to 8 rows go through
+    lutgemm_compute_shift_scale_pow2 (here, with the option at 2, onto the block-scaled kernel);
+    an alpha that is no power of two, or other row counts, keep the ordinary entry."""
+    from shiftaddllm_amd.lut_gemm.quant import LutLinear
+    N, K, nb = 512, 1024, 3
+    bW, alpha, x, _ = _problem(N, K, nb, 8, seed=5)
+    lin = LutLinear(K, N, group_size=128, wbit=nb, bias=None, alpha_format="rowwise_fp16").to(gpu_device)
+    lin.binaryWeight.data = bW.to(gpu_device)
+    lin.alpha.data = alpha.to(gpu_device)
+    lib = native.cabi()
+    for M in (1, 4, 8):
+        xm = x[:M].contiguous()
+        want, _ = orc.gemv_rowwise_c(bW.numpy(), alpha.numpy(), xm.numpy(), K // 128)
+        got = lin(xm.to(gpu_device))
+        assert lin._alphas_are_powers_of_two()
+        rel, mad = orc.error_metrics(got.float().cpu().numpy(), want.astype(np.float32))
+        assert rel <= 2e-4 and mad <= 1e-3, (M, rel, mad)
+        direct = _run(lib.lutgemm_gemv_rowwise_pow2_f16, gpu_device, bW, alpha, xm, torch.zeros((M, N)).half())
+        assert torch.equal(got, direct)
+    # one alpha with a mantissa bit: the module notices (the tensor's version changed) and keeps the fp16 entry
+    lin.alpha.data[0, 0, 0] = 0.75 * lin.alpha.data[0, 0, 0]
+    lin.alpha.data = lin.alpha.data.clone()
+    assert not lin._alphas_are_powers_of_two()
+    a2 = lin.alpha.data.cpu()
+    xm = x[:4].contiguous()
+    want, _ = orc.gemv_rowwise_c(bW.numpy(), a2.numpy(), xm.numpy(), K // 128)
+    got = lin(xm.to(gpu_device))
+    rel, mad = orc.error_metrics(got.float().cpu().numpy(), want.astype(np.float32))
+    assert rel <= 2e-4 and mad <= 1e-3, (rel, mad)
+    assert torch.equal(got, _run(lib.lutgemm_gemv_rowwise_f16, gpu_device, bW, a2, xm, torch.zeros((4, N)).half()))
