@@ -58,7 +58,8 @@ def parse_args():
     ap.add_argument("--plain-only", action="store_true",
                     help="only the 224 launches one after the other (no branches, no fused sequences, no tables): for profiler runs")
     ap.add_argument("--profile-shape", type=str, default="",
-                    help="N,K[,nb[,iters[,M]]]: only launch this shape repeatedly (for rocprofv3 runs) and exit")
+                    help="N,K[,nb[,iters[,M[,1]]]]: only launch this shape repeatedly (for rocprofv3 runs) and exit; "
+                         "a sixth field of 1 goes through lutgemm_gemv_rowwise_pow2_f16")
     ap.add_argument("--profile-floor", type=str, default="",
                     help="N,K[,nb[,iters]]: only launch the floor kernels for this shape (empty launch; stream-read of the sign words) and exit")
     ap.add_argument("--profile-decode", type=int, default=0,
@@ -66,6 +67,9 @@ def parse_args():
     ap.add_argument("--profile-phases", type=str, default="",
                     help="N,K[,nb[,iters]] or 'chain': run the shape (or one chained Llama-2-7B block) on the time-stamped "
                          "build of the library and print where the time of a launch goes, then exit")
+    ap.add_argument("--mark-timed", action="store_true",
+                    help="launch the library's 16-byte copy kernel right before and after the timed replays of the "
+                         "224-launch step, so that a kernel trace can be cut down to exactly those launches")
     ap.add_argument("--profile-copy", type=int, default=0,
                     help="bytes: only run the calibration copy kernel a few times (for rocprofv3 --pmc) and exit")
     return ap.parse_args()
@@ -306,9 +310,11 @@ def main():
             fn()
         return gr
 
-    def timed(fn, gr, steps, warmup):
+    def timed(fn, gr, steps, warmup, mark=None):
         """(wall ms/step, device ms/step): wall clock between synchronisations and
-        HIP events recorded on the launch stream around the same region."""
+        HIP events recorded on the launch stream around the same region.  `mark`, if given, is
+        called right before and right after the timed region (it launches a marker kernel by which a
+        kernel trace can tell the timed launches from the others)."""
         def step():
             with torch.cuda.stream(stream):
                 if gr is not None:
@@ -318,6 +324,9 @@ def main():
         for _ in range(warmup):
             step()
         torch.cuda.synchronize()
+        if mark:
+            mark()
+            torch.cuda.synchronize()
         ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         t_start = time.perf_counter()
         with torch.cuda.stream(stream):
@@ -328,6 +337,9 @@ def main():
             ev1.record(stream)
         torch.cuda.synchronize()
         wall = (time.perf_counter() - t_start) * 1e3 / steps
+        if mark:
+            mark()
+            torch.cuda.synchronize()
         return wall, ev0.elapsed_time(ev1) / steps
 
     def us_per_call(seq_fn, n_calls, reps=3):
@@ -386,12 +398,17 @@ def main():
         nb = parts[2] if len(parts) > 2 else NB
         iters = parts[3] if len(parts) > 3 else 8
         rows = parts[4] if len(parts) > 4 else 1
+        pow2 = len(parts) > 5 and parts[5] == 1
         pool = [Gemv(torch, dev, N, K, nb, 100 + i, M=rows) for i in range(iters)]
         with torch.cuda.stream(stream):
             for g in pool:      # each launch touches weights never read before
-                run(g, sp)
+                if pow2:
+                    check(lib.lutgemm_gemv_rowwise_pow2_f16(*g.args(), sp))
+                else:
+                    run(g, sp)
         stream.synchronize()
-        print(json.dumps({"shape": [N, K, nb], "rows": rows, "launches": iters, "algorithmic_bytes_per_launch": alg_bytes(pool[0])}))
+        print(json.dumps({"shape": [N, K, nb], "rows": rows, "launches": iters, "pow2_entry": pow2,
+                          "algorithmic_bytes_per_launch": alg_bytes(pool[0])}))
         return
 
     # ---- weight pool: `layers` decoder blocks x 7 linears -----------------
@@ -500,7 +517,11 @@ def main():
                 graph_plain.replay() if graph_plain is not None else seq_plain()
         torch.cuda.synchronize()
     # ---- the timed step: 224 launches strictly one after the other --------------------
-    ms_per_step, dev_ms_per_step = timed(seq_plain, graph_plain, args.steps, args.warmup)
+    marker = None
+    if args.mark_timed:
+        mk = torch.zeros(32, dtype=torch.uint8, device=dev)
+        marker = lambda: check(lib.lutgemm_copy_bytes(vp(mk[16:]), vp(mk[:16]), 16, sp))
+    ms_per_step, dev_ms_per_step = timed(seq_plain, graph_plain, args.steps, args.warmup, mark=marker)
     step_kind = "one after the other on one stream"
     # ---- the same launches with the dependencies of a decoder block as graph branches ----
     branched = None
