@@ -112,8 +112,11 @@ int lutgemm_gemv_rowwise_f16(const uint32_t *bW, const void *alpha_f16, const vo
  * largest of its 32; smaller ones are cut off at 2^-25 of it); the three pieces of up to
  * 5 rows share the 16 columns of one instruction.  Accumulation is fp32, one rounding to
  * fp16 at the end, as in every other entry point.  An infinity or NaN among the activations
- * gives NaN in every output of its row.  Other calls run exactly as
- * lutgemm_gemv_rowwise_f16 does.  With an alpha that breaks the promise the result is that
+ * gives NaN in every output of its row.  Calls of up to 16 rows that take the fp16
+ * matrix-core kernel with long K extents per workgroup form their sign operands through
+ * the same kind of table and gfx950's scaled fp4 -> fp16 conversion (option
+ * LUTGEMM_OPTION_POW2_CONVERT): the same exact products as lutgemm_gemv_rowwise_f16,
+ * summed in another order.  Other calls run exactly as lutgemm_gemv_rowwise_f16 does.  With an alpha that breaks the promise the result is that
  * of the alpha with its mantissa bits cleared (zero counts as 2^-15).
  * The split activations (3 * M * K + K + M * K / 8 bytes) live in a second per-stream
  * buffer that grows like the accumulator workspace: make one call of each size before
@@ -307,6 +310,12 @@ int lutgemm_describe_pow2_plan(int N, int K, int nb, int groups, int M, lutgemm_
  *                   kernel 1 = where it is the faster one (few rows, large matrices),
  *                   2 = wherever it applies, 0 = never (the call then behaves like
  *                   lutgemm_gemv_rowwise_f16); default 1
+ *   POW2_CONVERT  : calls of lutgemm_gemv_rowwise_pow2_f16 that take the fp16 matrix-core
+ *                   kernel form its sign operands through an LDS table and the scaled
+ *                   fp4 -> fp16 conversion instruction (which applies a power-of-two alpha
+ *                   as its scale) instead of a shift and a bit operation per fp16 pair
+ *                   1 = where that is faster (up to 16 rows, six or more rounds of K-steps
+ *                   per workgroup), 2 = always, 0 = never; default 1
  *   CHAIN_GRID    : workgroups of a chained launch (0 = as many as the device holds
  *                   at once, which is also the upper limit)
  *   CHAIN_BLOCKS  : ranges the problems of one stage of a chained launch are cut into
@@ -322,7 +331,8 @@ int lutgemm_describe_pow2_plan(int N, int K, int nb, int groups, int M, lutgemm_
 #define LUTGEMM_OPTION_CHAIN_GRID 7
 #define LUTGEMM_OPTION_TWIN_ITEMS 8
 #define LUTGEMM_OPTION_BLOCK_SCALED 9
-#define LUTGEMM_OPTION_COUNT 10
+#define LUTGEMM_OPTION_POW2_CONVERT 10
+#define LUTGEMM_OPTION_COUNT 11
 int lutgemm_set_option(int which, int value);
 int lutgemm_get_option(int which);
 

@@ -6,10 +6,17 @@ namespace lutgemm {
 namespace {
 
 template <int NB>
-hipError_t launch_nb(const Problem &p, int mt, hipStream_t stream)
+hipError_t launch_nb(const Problem &p, int mt, bool pow2, hipStream_t stream)
 {
     const dim3 grid((unsigned)p.n_blocks), block(kMfmaThreads);
-    if (mt == 1 && p.sets_per_split == kMfmaWaves)  // one round per K-slice
+    const bool one = mt == 1 && p.sets_per_split == kMfmaWaves;  // one round per K-slice
+    if (pow2 && one)
+        hipLaunchKernelGGL((lut_gemm_mfma_kernel<NB, 1, true, true>), grid, block, 0, stream, p);
+    else if (pow2 && mt == 2)
+        hipLaunchKernelGGL((lut_gemm_mfma_kernel<NB, 2, false, true>), grid, block, 0, stream, p);
+    else if (pow2)
+        hipLaunchKernelGGL((lut_gemm_mfma_kernel<NB, 1, false, true>), grid, block, 0, stream, p);
+    else if (one)
         hipLaunchKernelGGL((lut_gemm_mfma_kernel<NB, 1, true>), grid, block, 0, stream, p);
     else if (mt == 2)
         hipLaunchKernelGGL((lut_gemm_mfma_kernel<NB, 2>), grid, block, 0, stream, p);
@@ -43,13 +50,13 @@ hipError_t launch_mfma_fused(const Problem &p, int mt, hipStream_t stream)
     }
 }
 
-hipError_t launch_mfma(const Problem &p, int mt, hipStream_t stream)
+hipError_t launch_mfma(const Problem &p, int mt, bool pow2, hipStream_t stream)
 {
     switch (p.nb) {
-    case 1: return launch_nb<1>(p, mt, stream);
-    case 2: return launch_nb<2>(p, mt, stream);
-    case 3: return launch_nb<3>(p, mt, stream);
-    default: return launch_nb<4>(p, mt, stream);
+    case 1: return launch_nb<1>(p, mt, pow2, stream);
+    case 2: return launch_nb<2>(p, mt, pow2, stream);
+    case 3: return launch_nb<3>(p, mt, pow2, stream);
+    default: return launch_nb<4>(p, mt, pow2, stream);
     }
 }
 

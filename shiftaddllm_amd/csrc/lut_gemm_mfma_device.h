@@ -49,8 +49,13 @@ constexpr int kMfmaStepK = 128;
 constexpr int kRedRow = 65;           // the final reduction's LDS rows, padded against bank conflicts
 template <int MT>
 constexpr int kMfmaRedBytes = kMfmaWaves * 16 * MT * kRedRow * 4;
-template <int MT>
-constexpr int kMfmaLdsBytes = kMfmaRedBytes<MT> + 16 * MT * 4;
+// POW2 instances keep a 64 KiB table in front (sign byte -> eight 4-bit floats, see mfma_tile); the
+// final reduction takes its place afterwards, the rows' reciprocal RMS sit behind both.
+constexpr int kSignLutBytes = 256 * 64 * 4;   // 256 entries x 64 copies: copy l for lane l, one bank per lane of a half-wave
+template <int MT, bool POW2 = false>
+constexpr int kMfmaScaleOffset = (POW2 && kSignLutBytes > kMfmaRedBytes<MT>) ? kSignLutBytes : kMfmaRedBytes<MT>;
+template <int MT, bool POW2 = false>
+constexpr int kMfmaLdsBytes = kMfmaScaleOffset<MT, POW2> + 16 * MT * 4;
 
 // Operands of one K-step of a wave: per bit plane word kb of 4 outputs; the alphas of
 // those 4 outputs for bit plane kb (one load covers all planes: lane group kb of the wave
@@ -99,12 +104,20 @@ __device__ __forceinline__ f16x8 expand_signs(uint32_t w, int beta, uint32_t alp
     return __builtin_bit_cast(f16x8, r);
 }
 
-// xs: kMfmaLdsBytes<MT> bytes of LDS for the final reduction (and, behind them, the
+// xs: kMfmaLdsBytes<MT, POW2> bytes of LDS for the final reduction (and, behind them, the
 // reciprocal RMS of the tile's rows).
 // EXTRA: the launch honours the split-RMSNorm fields of the problem (next_in, sumsq_*).
 // ONE: every K-slice of the launch is a single round, i.e. a wave takes at most one step (the
 //      host's choice): nothing is requested beyond that step.
-template <int NB, int MT, bool EXTRA = false, bool ONE = false>
+// POW2: the caller promises that every alpha is a positive normal fp16 power of two.  Sign bits then
+//      become fp16 +-alpha without the per-pair shift and bit operation: a byte of the sign word
+//      (eight signs) indexes a table in LDS whose entries hold eight 4-bit floats +-1 (e2m1 codes
+//      0x2 / 0xA), and v_cvt_scalef32_pk_f16_fp4 turns two of them into a packed fp16 pair times a
+//      scale of which the hardware uses the exponent only (measured: scale 3.0 gives +-2), which for
+//      a power of two is the alpha itself.  One table read and four conversions per matrix
+//      instruction instead of eight vector operations, the eight signs come out in input order, so
+//      the activations need no permutes either.
+template <int NB, int MT, bool EXTRA = false, bool ONE = false, bool POW2 = false>
 __device__ __forceinline__ void mfma_tile(const Problem &p, int local_block, char *xs)
 {
     const int tid = threadIdx.x;
@@ -135,7 +148,7 @@ __device__ __forceinline__ void mfma_tile(const Problem &p, int local_block, cha
     // The slots are requested here, ahead of everything else, and summed once the first
     // step's operands have been requested behind them (see the main loop): loads return in
     // order, so that wait is for the slots alone.
-    float *row_scale = (float *)(xs + kMfmaRedBytes<MT>);
+    float *row_scale = (float *)(xs + kMfmaScaleOffset<MT, POW2>);
     typedef float f32x4v __attribute__((ext_vector_type(4)));
     constexpr int kScaleRows = 2 * MT;  // rows per wave
     bool scaled = false;
@@ -174,6 +187,24 @@ __device__ __forceinline__ void mfma_tile(const Problem &p, int local_block, cha
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) acc[e][mt] = (f32x4){0.0f, 0.0f, 0.0f, 0.0f};
 
+    // POW2: the sign table.  Entry i, copy c at byte i * 256 + 4 * c; lane l reads copy l, so one
+    // v_perm_b32 of (sign word, per-lane constant) is the address: index byte in bits 8..15, the
+    // lane's copy offset in bits 0..7.
+    [[maybe_unused]] const uint32_t lane_off = (uint32_t)(4 * lane) * 0x01010101u;
+    if constexpr (POW2) {
+        uint32_t *lut = (uint32_t *)xs;
+#pragma unroll 4
+        for (int idx = tid; idx < kSignLutBytes / 4; idx += kMfmaThreads) {   // a wave writes one entry's 64 copies
+            // (the entry index is the same for the whole wave: scalar arithmetic)
+            uint32_t v = (uint32_t)__builtin_amdgcn_readfirstlane(idx >> 6);   // bit j of it -> bit 4 * j + 3
+            v = (v | (v << 12)) & 0x000f000fu;
+            v = (v | (v << 6)) & 0x03030303u;
+            v = (v | (v << 3)) & 0x11111111u;
+            lut[idx] = 0xaaaaaaaau ^ (v << 3);
+        }
+        __syncthreads();
+    }
+
     auto compute = [&](const MfmaOperands<NB, MT> &ops) {
 #pragma unroll
         for (int b = 0; b < NB; ++b) {
@@ -181,6 +212,33 @@ __device__ __forceinline__ void mfma_tile(const Problem &p, int local_block, cha
             const int from = 4 * (16 * b + li);   // the lane of group b that holds this lane's outputs
             const u32x2 al = {(uint32_t)__builtin_amdgcn_ds_bpermute(from, (int)ops.alpha.x),
                               (uint32_t)__builtin_amdgcn_ds_bpermute(from, (int)ops.alpha.y)};
+            if constexpr (POW2) {
+                // the alpha of output e as the conversion's fp32 scale
+                const float scale[4] = {half_bits_to_float(al.x & 0xffffu), half_bits_to_float(al.x >> 16),
+                                        half_bits_to_float(al.y & 0xffffu), half_bits_to_float(al.y >> 16)};
+                constexpr uint32_t sel[4] = {0x0c0c0400u, 0x0c0c0501u, 0x0c0c0602u, 0x0c0c0703u};
+#pragma unroll
+                for (int beta = 0; beta < 4; ++beta) {
+                    // byte beta of the sign word = inputs 8 * beta .. + 7 of the lane's 32, in order
+                    f16x8 bx[MT];
+#pragma unroll
+                    for (int mt = 0; mt < MT; ++mt) bx[mt] = __builtin_bit_cast(f16x8, ops.x[mt][beta]);
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const uint32_t nib = *(const uint32_t *)(xs + __builtin_amdgcn_perm(w4[e], lane_off, sel[beta]));
+                        typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+                        const f16x2 p0 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(nib, scale[e], 0);
+                        const f16x2 p1 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(nib, scale[e], 1);
+                        const f16x2 p2 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(nib, scale[e], 2);
+                        const f16x2 p3 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(nib, scale[e], 3);
+                        const f16x8 a = {p0[0], p0[1], p1[0], p1[1], p2[0], p2[1], p3[0], p3[1]};
+#pragma unroll
+                        for (int mt = 0; mt < MT; ++mt)
+                            acc[e][mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, bx[mt], acc[e][mt], 0, 0, 0);
+                    }
+                }
+                continue;
+            }
             // the alpha of output e in both halves of a register
             const uint32_t a2[4] = {__builtin_amdgcn_perm(al.x, al.x, 0x01000100u), __builtin_amdgcn_perm(al.x, al.x, 0x03020302u),
                                     __builtin_amdgcn_perm(al.y, al.y, 0x01000100u), __builtin_amdgcn_perm(al.y, al.y, 0x03020302u)};
@@ -258,6 +316,7 @@ __device__ __forceinline__ void mfma_tile(const Problem &p, int local_block, cha
     // ---- the 8 waves' accumulators meet in LDS -----------------------------------
     // red[wave][j = (e*MT + mt)*4 + r][lane], rows padded to 65 words so that the
     // read-out below (consecutive threads = consecutive outputs) spreads over the banks
+    if constexpr (POW2) __syncthreads();   // (the table's memory: every wave is done with it)
     float *red = (float *)xs;
 #pragma unroll
     for (int e = 0; e < 4; ++e)
@@ -328,11 +387,11 @@ __device__ __forceinline__ void mfma_tile(const Problem &p, int local_block, cha
     }
 }
 
-template <int NB, int MT, bool ONE = false>
+template <int NB, int MT, bool ONE = false, bool POW2 = false>
 __global__ void __launch_bounds__(kMfmaThreads) lut_gemm_mfma_kernel(const Problem p)
 {
-    __shared__ __attribute__((aligned(16))) char xs[kMfmaLdsBytes<MT>];
-    mfma_tile<NB, MT, false, ONE>(p, (int)blockIdx.x, xs);
+    __shared__ __attribute__((aligned(16))) char xs[kMfmaLdsBytes<MT, POW2>];
+    mfma_tile<NB, MT, false, ONE, POW2>(p, (int)blockIdx.x, xs);
 }
 
 // One problem with the split-RMSNorm fields honoured.

@@ -178,7 +178,7 @@ constexpr Option kOptions[LUTGEMM_OPTION_COUNT] = {
     {"LUTGEMM_TARGET_BLOCKS", 0}, {"LUTGEMM_FIRST_SHARE", 60}, {"LUTGEMM_MFMA_MIN_M", 3},
     {"LUTGEMM_MFMA_BLOCKS", 0},   {"LUTGEMM_PAIR_TABLES", 1},  {"LUTGEMM_SINGLE_ITEM", 1},
     {"LUTGEMM_CHAIN_BLOCKS", 0}, {"LUTGEMM_CHAIN_GRID", 0},  {"LUTGEMM_TWIN_ITEMS", 4},
-    {"LUTGEMM_BLOCK_SCALED", 1},
+    {"LUTGEMM_BLOCK_SCALED", 1}, {"LUTGEMM_POW2_CONVERT", 1},
 };
 std::atomic<int> g_option[LUTGEMM_OPTION_COUNT];
 std::once_flag g_option_once;
@@ -444,7 +444,7 @@ int run_mfma(Problem &p, const Accum &acc)
         int rc = accum_words(acc, (size_t)p.M * p.N, &p.accum);
         if (rc != LUTGEMM_OK) return rc;
     }
-    const hipError_t e = launch_mfma(p, mt, acc.stream);
+    const hipError_t e = launch_mfma(p, mt, false, acc.stream);
     return e == hipSuccess ? LUTGEMM_OK : hip_fail(e);
 }
 
@@ -574,6 +574,22 @@ bool mx_wanted(const Problem &p)
     return (p.M <= 5 && sign_bytes >= (48l << 20)) || (p.M <= 8 && sign_bytes >= (96l << 20));
 }
 
+// Whether a planned fp16 matrix-core launch whose alphas are powers of two should form its sign
+// operands through the LDS table and the scaled fp4 -> fp16 conversion (5 vector instructions per
+// matrix instruction instead of 10) rather than by shift and bit operation.  The table costs every
+// workgroup a 64 KiB build and a barrier (1 to 2 us), which pays from about six rounds of K-steps per
+// workgroup on; the 32-row tile would drop to one workgroup per CU with the table and loses.
+// Measured (us, shift-and-bit form vs converted form, 16 rows): 28672x8192x4 48.9 / 42.6,
+// 8192x28672x4 48.2 / 42.8, 28672x8192x2 30.0 / 28.6 (8 rows 28.4 / 25.0); 8192x8192x4 (2 rounds) 19.6 / 19.4,
+// 11008x4096x3 (4 rounds) 15.0 / 15.8, 4096x4096x3 (1 round) 8.8 / 11.0; 32 rows 28672x8192x4 74.1 / 77.6.
+// Option POW2_CONVERT: 1 = by this rule, 2 = whenever the promise is given, 0 = never.
+bool convert_wanted(const Problem &p, int mt)
+{
+    const int how = option(LUTGEMM_OPTION_POW2_CONVERT);
+    if (how != 1) return how == 2;
+    return mt == 1 && p.sets_per_split >= 6 * kMfmaWaves;
+}
+
 // Row-wise problem whose alphas are powers of two, with enough rows for the matrix cores: the
 // block-scaled kernel (16-row tiles; more rows are further row chunks that stream the same sign
 // words side by side).
@@ -608,7 +624,7 @@ int run(int mode, const uint32_t *bW, const void *alpha, const void *qbias, cons
     }
     hipError_t e;
     if (kernel == kMatrixCore)
-        e = launch_mfma(p, mrows / 16, acc.stream);
+        e = launch_mfma(p, mrows / 16, alpha_pow2 && convert_wanted(p, mrows / 16), acc.stream);
     else if (mode == kRowF16 || mode == kUniformF16)
         e = launch_gemv_rowwise(p, mode, mrows, acc.stream);
     else if (p.rows_per_group >= kTileCols)  // a tile spans at most two row groups

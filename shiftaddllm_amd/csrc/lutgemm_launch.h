@@ -24,7 +24,8 @@ hipError_t launch_gemv_chain(const Chain &c, int blocks, hipStream_t stream);
 // workgroups of that kernel the current device holds at once (looked up once per device)
 hipError_t chain_resident_workgroups(int *count);
 // matrix-core kernel; mt = 1 (16-row tiles) or 2 (32-row tiles)
-hipError_t launch_mfma(const Problem &p, int mt, hipStream_t stream);
+// pow2: the caller promises power-of-two alphas (signs through the LDS table and the fp4 conversion)
+hipError_t launch_mfma(const Problem &p, int mt, bool pow2, hipStream_t stream);
 hipError_t launch_mfma_fused(const Problem &p, int mt, hipStream_t stream);  // one problem with fused extras
 hipError_t launch_mfma_group(const Group &g, int mt, int blocks, hipStream_t stream);
 // block-scaled matrix-core kernel (alphas are powers of two): splits p.x into `split` (mx_split_bytes:

@@ -56,7 +56,7 @@ C_ABI_SYMBOLS = (
 
 MAX_GROUP = 8
 OPTIONS = {"TARGET_BLOCKS": 0, "FIRST_SHARE": 1, "MFMA_MIN_M": 2, "MFMA_BLOCKS": 3, "PAIR_TABLES": 4, "SINGLE_ITEM": 5,
-           "CHAIN_BLOCKS": 6, "CHAIN_GRID": 7, "TWIN_ITEMS": 8, "BLOCK_SCALED": 9}
+           "CHAIN_BLOCKS": 6, "CHAIN_GRID": 7, "TWIN_ITEMS": 8, "BLOCK_SCALED": 9, "POW2_CONVERT": 10}
 CHAIN_MAX_ROWS = 4
 CHAIN_MAX_TAG = 65534
 NOALLOC_MAX_WORDS = 1 << 18

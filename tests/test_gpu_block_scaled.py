@@ -23,6 +23,7 @@ def _block_scaled_wherever_it_applies():
     lib.lutgemm_set_option(which, 2)
     yield
     lib.lutgemm_set_option(which, -1)
+    lib.lutgemm_set_option(native.OPTIONS["POW2_CONVERT"], -1)
 
 
 def _ptr(t):
@@ -108,6 +109,7 @@ def test_pow2_entry_point_falls_back_where_the_block_scaled_kernel_does_not_appl
         assert torch.equal(a, b), (N, K, nb, M, group)
     which = native.OPTIONS["BLOCK_SCALED"]
     lib.lutgemm_set_option(which, 0)
+    lib.lutgemm_set_option(native.OPTIONS["POW2_CONVERT"], 0)
     try:
         bW, alpha, x, bias = _problem(2048, 1024, 3, 8, seed=3)
         a = _run(lib.lutgemm_gemv_rowwise_pow2_f16, gpu_device, bW, alpha, x, bias)
@@ -115,6 +117,7 @@ def test_pow2_entry_point_falls_back_where_the_block_scaled_kernel_does_not_appl
         assert torch.equal(a, b)
     finally:
         lib.lutgemm_set_option(which, 2)
+        lib.lutgemm_set_option(native.OPTIONS["POW2_CONVERT"], -1)
 
 
 def test_default_rule_takes_the_block_scaled_kernel_for_few_rows_of_a_large_matrix(gpu_device):
@@ -166,3 +169,32 @@ def test_lutlinear_takes_the_pow2_entry_for_a_few_rows(gpu_device):
     rel, mad = orc.error_metrics(got.float().cpu().numpy(), want.astype(np.float32))
     assert rel <= 2e-4 and mad <= 1e-3, (rel, mad)
     assert torch.equal(got, _run(lib.lutgemm_gemv_rowwise_f16, gpu_device, bW, a2, xm, torch.zeros((4, N)).half()))
+
+
+@pytest.mark.parametrize("N,K,nb,M,group", [
+    (256, 256, 1, 3, 128), (1024, 1024, 2, 4, 128), (4096, 4096, 3, 16, 128), (2048, 1024, 4, 17, 128),
+    (528, 512, 3, 5, 256), (1040, 2048, 4, 33, 512), (11008, 4096, 3, 8, 128), (4096, 11008, 2, 32, 128),
+    (64, 128, 4, 16, 128), (16, 1024, 2, 7, 128), (8192, 8192, 4, 16, 128)])
+def test_fp16_matrix_core_kernel_with_converted_sign_operands(gpu_device, N, K, nb, M, group):
+    """With the block-scaled kernel switched off, a pow2 call takes the fp16 matrix-core kernel whose sign
+    operands come from the LDS table and the scaled fp4 -> fp16 conversion (option POW2_CONVERT, default
+    1 = where it is faster, 2 = always): the same exact products as the shift-and-bit-operation form,
+    summed in another order, so the two agree to a rounding of the fp32 sums; and the oracle's result.
+    With the option at 0 the call is lutgemm_gemv_rowwise_f16 bit for bit."""
+    lib = native.cabi()
+    lib.lutgemm_set_option(native.OPTIONS["BLOCK_SCALED"], 0)
+    lib.lutgemm_set_option(native.OPTIONS["POW2_CONVERT"], 2)
+    print(f"converted signs N={N} K={K} nb={nb} M={M} group={group}", flush=True)
+    bW, alpha, x, bias = _problem(N, K, nb, M, seed=N + K + nb + M, group=group)
+    want, _ = orc.gemv_rowwise_c(bW.numpy(), alpha.numpy(), x.numpy(), K // group, out=bias.numpy())
+    got = _run(lib.lutgemm_gemv_rowwise_pow2_f16, gpu_device, bW, alpha, x, bias, group)
+    rel, mad = orc.error_metrics(got.float().cpu().numpy(), want.astype(np.float32))
+    assert rel <= 2e-4 and mad <= 1e-3, (rel, mad)
+    other = _run(lib.lutgemm_gemv_rowwise_f16, gpu_device, bW, alpha, x, bias, group)
+    assert torch.allclose(got.float(), other.float(), rtol=2e-3, atol=2e-3 * float(other.float().abs().max()))
+    which = native.OPTIONS["POW2_CONVERT"]
+    lib.lutgemm_set_option(which, 0)
+    try:
+        assert torch.equal(_run(lib.lutgemm_gemv_rowwise_pow2_f16, gpu_device, bW, alpha, x, bias, group), other)
+    finally:
+        lib.lutgemm_set_option(which, -1)
