@@ -198,3 +198,48 @@ def test_fp16_matrix_core_kernel_with_converted_sign_operands(gpu_device, N, K, 
         assert torch.equal(_run(lib.lutgemm_gemv_rowwise_pow2_f16, gpu_device, bW, alpha, x, bias, group), other)
     finally:
         lib.lutgemm_set_option(which, -1)
+
+
+@pytest.mark.parametrize("block_scaled,convert", [(2, 0), (0, 2), (1, 1)])
+def test_random_shapes_of_the_pow2_entry_against_a_dense_product(gpu_device, block_scaled, convert):
+    """90 seeded random problems per setting (K % 128, N % 16, group sizes from 128 up, 1-4 bit planes,
+    3-40 rows, power-of-two alphas over nine binades, activations of mixed magnitude, a bias in `out`)
+    through lutgemm_gemv_rowwise_pow2_f16 with the block-scaled kernel forced, with the converted
+    sign operands forced, and under the default rules, against the dense fp64 product of the
+    dequantised matrix formed on the GPU by framework operations."""
+    import random
+    dev = gpu_device
+    lib = native.cabi()
+    lib.lutgemm_set_option(native.OPTIONS["BLOCK_SCALED"], block_scaled)
+    lib.lutgemm_set_option(native.OPTIONS["POW2_CONVERT"], convert)
+    rng = random.Random(77 + 10 * block_scaled + convert)
+    plan = native.Plan()
+    kernels = set()
+    for case in range(90):
+        K = 128 * rng.randint(1, 72)
+        N = 16 * rng.randint(1, 520)
+        gs = rng.choice([g for g in (128, 256, 512, 1024, K) if K % g == 0])
+        nb = rng.randint(1, 4)
+        M = rng.choice((3, 4, 5, 6, 8, 9, 13, 16, 17, 24, 32, 33, 40))
+        g = torch.Generator(device=dev).manual_seed(1000 + case)
+        bW = torch.randint(-2 ** 31, 2 ** 31 - 1, (K // 32, nb, N), generator=g, device=dev, dtype=torch.int32)
+        e = torch.randint(-13, -4, (K // gs, nb, N), generator=g, device=dev).float()
+        alpha = torch.exp2(e).half()
+        x = torch.randn((M, K), generator=g, device=dev)
+        if case % 3 == 0:
+            x = x * torch.exp2(torch.randint(-8, 3, (M, K), generator=g, device=dev).float())
+        x = x.half()
+        bias = torch.randn((M, N), generator=g, device=dev).half()
+        out = bias.clone()
+        rc = lib.lutgemm_gemv_rowwise_pow2_f16(_ptr(bW), _ptr(alpha), _ptr(x), _ptr(out), N, K, nb, K // gs, M, _sp())
+        assert rc == 0, lib.lutgemm_strerror(rc).decode()
+        torch.cuda.synchronize()
+        signs = ((bW.unsqueeze(1) >> torch.arange(32, device=dev).view(1, 32, 1, 1)) & 1).double() * 2 - 1
+        Wq = (signs.reshape(K, nb, N) * alpha.double().repeat_interleave(gs, dim=0)).sum(1)      # [K][N]
+        want = bias.double() + x.double() @ Wq
+        rel = ((out.double() - want).norm() / want.norm()).item()
+        mad = ((out.double() - want).abs().max() / want.abs().max()).item()
+        assert lib.lutgemm_describe_pow2_plan(N, K, nb, K // gs, M, ctypes.byref(plan)) == 0
+        kernels.add(plan.kernel)
+        assert rel <= 5e-4 and mad <= 2.5e-3, (N, K, nb, gs, M, rel, mad)
+    assert kernels == ({2} if block_scaled == 2 else {1}), kernels
