@@ -569,6 +569,7 @@ void plan_mx(Problem &p)
 bool mx_wanted(const Problem &p)
 {
     const int how = option(LUTGEMM_OPTION_BLOCK_SCALED);
+    if ((long)p.M * p.K >= (1l << 30)) return false;   // (the split kernel indexes the activations with 32 bits)
     if (how != 1) return how == 2;
     const long sign_bytes = (long)p.N * (p.K / 8) * p.nb;
     return (p.M <= 5 && sign_bytes >= (48l << 20)) || (p.M <= 8 && sign_bytes >= (96l << 20));
