@@ -955,6 +955,12 @@ def main():
         if isinstance(v, dict):
             roof[f"decode_{k}_tokens_per_s"] = v["tokens_per_s"]
             roof[f"decode_{k}_ms_per_token"] = v["median_ms_per_token"]
+    # the largest small-batch shape (Llama-2-70B gate/up, 4-bit): microseconds per call by row count
+    c5 = (configs or {}).get("config5_llama70b", {}).get("28672x8192x4bit")
+    if c5:
+        for m, e in c5.items():
+            roof[f"llama70b_28672x8192x4bit_{m}_us"] = e["us_per_call"]
+        roof["llama70b_28672x8192x4bit_M1_frac"] = c5["M1"]["frac_hbm_peak"]
     result["roofline"] = roof
     print(json.dumps(result))
 
