@@ -49,8 +49,8 @@ constexpr int kMxPieces = 3;
 constexpr int kMxLutBytes = 256 * 256;   // 256 entries x 64 copies x 4 bytes: copy l % 64 for lane l, one bank each
 
 // ---- activations: fp16 -> three e4m3 pieces and a scale word per block of 32 ---------------------
-// One thread per (row, block of 32 consecutive inputs).  The pieces of a 128-input step are stored in
-// the order the B operand wants them (see above): the bytes a lane loads are contiguous.
+// Eight threads per (row, block of 32 consecutive inputs).  The pieces of a 128-input step are stored
+// in the order the B operand wants them (see above): the bytes a lane loads are contiguous.
 //   pieces: [3][M][K] bytes; within each 128-input step, block q's inputs 0..15 go to byte
 //           32 * (2 * (q & 1)) + 16 * (q >> 1), its inputs 16..31 to byte 32 * (2 * (q & 1) + 1) + 16 * (q >> 1);
 //           behind them one row of K zero bytes;
